@@ -36,13 +36,15 @@ def config_class(name):
 def config_from_dict(d):
     archs = d.get("architectures") or []
     names = list(archs[:1]) + ([d["model_type"]] if "model_type" in d else [])
+    if isinstance(d.get("architecture"), str):       # some families name theirs under this key, as one string
+        names.append(d["architecture"])
     if not names:
-        raise ConfigError("config.json has neither 'architectures' nor 'model_type'; registered: %s"
+        raise ConfigError("config.json has neither 'architectures' nor 'model_type' nor 'architecture'; registered: %s"
                           % ", ".join(registered_architectures()))
     for n in names:
         if n in _ARCHITECTURES:
             return _ARCHITECTURES[n].from_dict(d)
-    raise ConfigError("unknown architecture %s (from config.json 'architectures'/'model_type'); "
+    raise ConfigError("unknown architecture %s (from config.json 'architectures'/'model_type'/'architecture'); "
                       "registered: %s" % (" / ".join(map(repr, names)),
                                           ", ".join(registered_architectures())))
 

@@ -75,6 +75,57 @@ int ga_silu_mul(void* out, const void* gu, int tokens, int inter, int is_bf16, h
 // the same on a product that lies transposed, gu_t [2 inter, tokens] bfloat16; tokens and inter multiples of 8
 int ga_silu_mul_transposed(void* out, const void* gu_t, int tokens, int inter, hipStream_t stream);
 
+// a gated activation with bounded factors: out = g * sigmoid(alpha g) * (u + shift), g = min(gu[:, :inter], limit),
+// u = clamp(gu[:, inter:], -limit, limit)
+int ga_clamped_glu(void* out, const void* gu, int tokens, int inter, float limit, float alpha, float shift, int is_bf16,
+                   hipStream_t stream);
+
+// ---- scalar_norm.hip: RMS norm with ONE gain for all coordinates (gain: one float or bfloat16).  rows: out [num_rows,
+// hidden] = norm of the rows x[rows[r]] of the float stream (rows null: all rows in order).  add: residual float
+// [tokens, hidden] += norm(y); copy (or null): the new residual in y's dtype
+int ga_scalar_rmsnorm_rows(void* out, const void* x, const void* gain, const void* rows, int num_rows, int hidden, float eps,
+                           int out_bf16, int gain_bf16, hipStream_t stream);
+int ga_add_scalar_rmsnorm(void* residual, const void* y, const void* gain, void* copy, int tokens, int hidden, float eps,
+                          int y_bf16, int gain_bf16, hipStream_t stream);
+
+// ---- embedding_sinusoid.hip: out float [tokens, hidden] = table[ids] + (sin | cos)(position * freq[i / 2]), then the norm
+// with one gain (gain null: no norm); freq float [(hidden + 1) / 2]
+int ga_embedding_sinusoid_norm(void* out, const void* table, const void* ids, const void* positions, const void* freq,
+                               const void* gain, int tokens, int hidden, float eps, int table_bf16, int gain_bf16,
+                               hipStream_t stream);
+
+// ---- short_conv.hip: causal convolution of `taps` taps over time on each channel of the float stream x [tokens, width],
+// w float [width, taps]; the inputs before a step's tokens come from state float [slots, taps - 1, width].  apply: out
+// (compute dtype) = (add_input ? x : 0) + conv(x); update (after apply): the state moves on by the step's tokens.
+// slots int64 [entries], token_entry int32 [tokens], cu int32 [entries + 1], q_start int32 [entries]
+int ga_short_conv_apply(void* out, const void* x, const void* w, const void* state, const void* slots,
+                        const void* token_entry, const void* cu, const void* q_start, int tokens, int width, int taps,
+                        int add_input, int out_bf16, hipStream_t stream);
+int ga_short_conv_update(void* state, const void* x, const void* slots, const void* cu, const void* q_start, int entries,
+                         int width, int taps, hipStream_t stream);
+
+// ---- gated_recurrence.hip: the HGRN2 recurrence.  proj float [tokens, 2 heads dim + heads vdim] (row stride given) holds
+// (q before its SiLU | forget-gate logits | v); state float [slots, heads, dim, vdim]; out float [tokens, heads, vdim]
+int ga_hgrn2_scan(void* out, const void* proj, int64_t proj_stride, const void* f_bias, const void* lower, void* state,
+                  const void* slots, const void* cu, const void* q_start, int entries, int heads, int dim, int vdim,
+                  hipStream_t stream);
+// out [rows, vdim] (compute dtype) = x / sqrt(mean(x^2) + eps) * weight, x float [rows, vdim], weight float [vdim]
+int ga_headwise_rmsnorm(void* out, const void* x, const void* weight, int64_t rows, int vdim, float eps, int out_bf16,
+                        hipStream_t stream);
+
+// ---- latent_attention.hip: attention over a cached latent (one row c of `rank` numbers per token, in pages
+// [pages, page_size * rank]) that serves every head as key and as value; queries qa float, already in the latent space
+// (element strides per token and per head); window 0: all earlier keys; sink float [heads] or null; gate float
+// [tokens, heads] or null; out in the compute dtype (element strides per token and per head)
+int ga_latent_attention_max_rank();
+int ga_latent_prepare(void* cq, void* c_pages, void* gate, const void* proj, int64_t proj_stride, const void* wq,
+                      const void* wkv, const void* slot_mapping, int tokens, int q_rank, int kv_rank, int heads, float eps,
+                      int write_c, int is_bf16, hipStream_t stream);
+int ga_latent_attention(void* out, int64_t out_t, int64_t out_h, const void* qa, int64_t qa_t, int64_t qa_h,
+                        const void* c_pages, const void* block_table, int table_width, const void* token_entry,
+                        const void* positions, const void* sink, const void* gate, int tokens, int heads, int rank,
+                        int page_size, int window, float scale, int is_bf16, hipStream_t stream);
+
 // ---- attention_generic.hip: every token attends to its request's pages; any head size up to 256, window or 0;
 // tokens_per_workgroup neighbouring tokens share a workgroup's tiles of keys and values (0: the library chooses; -1: the
 // same, and every request of the step has at least 8 tokens in it); few_tokens_workgroups, fill_workgroups: the two

@@ -281,6 +281,8 @@ class ModelRunner:
         buf.fill(host)
         cache, ps = self.cache, self.page_size
         def view(owner, place, spec, owns):
+            if spec is None:             # a place in a block's list that keeps nothing in this layer
+                return None
             if isinstance(spec, StateSpec):
                 return StateView(cache.state_tensors[(owner, place)], buf.dev["state_slots"], owns)
             gi, _ = cache.group_of[(owner, place)]

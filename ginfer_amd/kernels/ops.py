@@ -748,3 +748,205 @@ def paged_attention(q, k_pages, v_pages, block_table, step, num_heads, num_kv_he
         grouping = 0
     return paged_attention_generic(q, k_pages, v_pages, block_table, step.token_entry, step.positions, num_heads,
                                    num_kv_heads, head_dim, scale, window, tokens_per_workgroup=grouping)
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# norm with one gain, embedding with sinusoidal positions, short convolution, gated recurrence, latent attention
+
+def _f32(t, shape, name):
+    _need(t is not None and t.dtype == torch.float32 and tuple(t.shape) == tuple(shape) and t.is_contiguous(),
+          "%s must be contiguous float32 %s", name, tuple(shape))
+
+
+def _scalar_gain(gain):
+    _need(gain.numel() == 1 and gain.dtype in (torch.float32, torch.bfloat16), "the gain must be one float32 or bfloat16 number")
+    return 1 if gain.dtype == torch.bfloat16 else 0
+
+
+def clamped_glu(gate_up, limit, alpha, shift, out=None):
+    """gate_up [T, 2I] -> [T, I]: g * sigmoid(alpha g) * (u + shift) with g = min(gate, limit), u = clamp(up, -limit, limit)."""
+    _dev(gate_up, out)
+    _need(gate_up.dim() == 2 and gate_up.is_contiguous() and gate_up.shape[1] % 2 == 0, "gate_up must be contiguous [T, 2I]")
+    T, I = gate_up.shape[0], gate_up.shape[1] // 2
+    if out is None:
+        out = torch.empty((T, I), dtype=gate_up.dtype, device=gate_up.device)
+    _need(out.dtype == gate_up.dtype and out.shape == (T, I) and out.is_contiguous(), "out must be contiguous [T, I]")
+    lib = build.load("activation")
+    _check(lib.ga_clamped_glu(_ptr(out), _ptr(gate_up), _i(T), _i(I), _f(limit), _f(alpha), _f(shift),
+                              _i(_is_bf16(gate_up.dtype)), _stream()), "clamped_glu")
+    return out
+
+
+def scalar_rmsnorm_rows(x, gain, eps, dtype, rows=None):
+    """x float32 [T, H]; gain: one number; rows int32 [R] or None -> [R or T, H] in `dtype`: g * x / sqrt(mean(x^2) + eps)."""
+    _dev(x, gain, rows)
+    _need(x.dtype == torch.float32 and x.dim() == 2 and x.is_contiguous(), "x must be contiguous float32 [T, H]")
+    T, H = x.shape
+    R = T
+    if rows is not None:
+        _need(rows.dtype == torch.int32 and rows.dim() == 1 and rows.is_contiguous(), "rows must be contiguous int32 [R]")
+        R = rows.shape[0]
+    out = torch.empty((R, H), dtype=dtype, device=x.device)
+    lib = build.load("scalar_norm")
+    _check(lib.ga_scalar_rmsnorm_rows(_ptr(out), _ptr(x), _ptr(gain), _ptr(rows), _i(R), _i(H), _f(eps), _i(_is_bf16(dtype)),
+                                      _i(_scalar_gain(gain)), _stream()), "scalar_rmsnorm_rows")
+    return out
+
+
+def add_scalar_rmsnorm(residual, y, gain, eps, copy=False):
+    """residual float32 [T, H] += g * y / sqrt(mean(y^2) + eps), in place; y [T, H] float32 or bfloat16.  With copy the
+    new residual also comes back in y's dtype (what the next product reads); for a float32 y that is the residual itself."""
+    _dev(residual, y, gain)
+    _need(residual.dtype == torch.float32 and residual.dim() == 2 and residual.is_contiguous(),
+          "residual must be contiguous float32 [T, H]")
+    _need(y.shape == residual.shape and y.is_contiguous(), "y must be contiguous %s, got %s", tuple(residual.shape), tuple(y.shape))
+    T, H = residual.shape
+    out = None
+    if copy and y.dtype != torch.float32:
+        out = torch.empty((T, H), dtype=y.dtype, device=y.device)
+    lib = build.load("scalar_norm")
+    _check(lib.ga_add_scalar_rmsnorm(_ptr(residual), _ptr(y), _ptr(gain), _ptr(out), _i(T), _i(H), _f(eps), _i(_is_bf16(y.dtype)),
+                                     _i(_scalar_gain(gain)), _stream()), "add_scalar_rmsnorm")
+    if not copy:
+        return None
+    return out if out is not None else residual
+
+
+def embedding_sinusoid_norm(table, ids, positions, freq, gain, eps):
+    """table [V, H], ids and positions int32 [T], freq float32 [(H + 1) // 2], gain: one number or None -> float32 [T, H]."""
+    _dev(table, ids, positions, freq, gain)
+    _need(table.dim() == 2 and table.is_contiguous(), "embedding table must be contiguous [V, H]")
+    T, H = ids.shape[0], table.shape[1]
+    for name, a in (("ids", ids), ("positions", positions)):
+        _need(a.dtype == torch.int32 and a.shape == (T,) and a.is_contiguous(), "%s must be contiguous int32 [T]", name)
+    _f32(freq, ((H + 1) // 2,), "freq")
+    out = torch.empty((T, H), dtype=torch.float32, device=table.device)
+    lib = build.load("embedding_sinusoid")
+    _check(lib.ga_embedding_sinusoid_norm(_ptr(out), _ptr(table), _ptr(ids), _ptr(positions), _ptr(freq), _ptr(gain), _i(T),
+                                          _i(H), _f(eps), _i(_is_bf16(table.dtype)),
+                                          _i(_scalar_gain(gain) if gain is not None else 0), _stream()), "embedding_sinusoid_norm")
+    return out
+
+
+SHORT_CONV_MAX_TAPS = 16
+
+
+def short_conv(x, weight, state, slots, step, dtype, add_input=True, update=True):
+    """x float32 [T, W] (the residual stream); weight float32 [W, taps]; state float32 [slots, taps - 1, W] (None for one
+    tap); slots int64 [entries].  Returns (x +) the causal convolution in `dtype`, the inputs before the step's tokens
+    taken from the state, and moves the state on by the step's tokens."""
+    _dev(x, weight, state, slots)
+    _need(x.dtype == torch.float32 and x.dim() == 2 and x.is_contiguous(), "x must be contiguous float32 [T, W]")
+    T, W = x.shape
+    _need(weight.dim() == 2 and weight.shape[0] == W and 1 <= weight.shape[1] <= SHORT_CONV_MAX_TAPS,
+          "the convolution's weight must be [%d, taps <= %d], got %s", W, SHORT_CONV_MAX_TAPS, tuple(weight.shape))
+    taps = weight.shape[1]
+    _f32(weight, (W, taps), "weight")
+    E = step.cu_tokens.shape[0] - 1
+    for name, a, n in (("token_entry", step.token_entry, T), ("cu_tokens", step.cu_tokens, E + 1), ("q_start", step.q_start, E)):
+        _need(a.dtype == torch.int32 and a.shape == (n,) and a.is_contiguous(), "%s must be contiguous int32 [%d]", name, n)
+    if taps > 1:
+        _need(state is not None and state.dtype == torch.float32 and state.dim() == 3 and state.is_contiguous()
+              and tuple(state.shape[1:]) == (taps - 1, W), "state must be contiguous float32 [slots, %d, %d]", taps - 1, W)
+        _need(slots.dtype == torch.int64 and slots.shape == (E,) and slots.is_contiguous(), "slots must be contiguous int64 [%d]", E)
+    out = torch.empty((T, W), dtype=dtype, device=x.device)
+    lib = build.load("short_conv")
+    _check(lib.ga_short_conv_apply(_ptr(out), _ptr(x), _ptr(weight), _ptr(state), _ptr(slots), _ptr(step.token_entry),
+                                   _ptr(step.cu_tokens), _ptr(step.q_start), _i(T), _i(W), _i(taps), _i(1 if add_input else 0),
+                                   _i(_is_bf16(dtype)), _stream()), "short_conv_apply")
+    if update and taps > 1:
+        _check(lib.ga_short_conv_update(_ptr(state), _ptr(x), _ptr(slots), _ptr(step.cu_tokens), _ptr(step.q_start), _i(E), _i(W),
+                                        _i(taps), _stream()), "short_conv_update")
+    return out
+
+
+HGRN2_MAX_DIM = 256
+
+
+def hgrn2_scan(proj, f_bias, lower, state, slots, step, heads, dim, vdim, update=True):
+    """proj float32 [T, 2 heads dim + heads vdim]: (q before its SiLU | forget-gate logits | v); f_bias, lower float32
+    [heads dim]; state float32 [slots, heads, dim, vdim], advanced in place.  Returns float32 [T, heads, vdim]."""
+    _dev(proj, f_bias, lower, state, slots)
+    T = proj.shape[0]
+    _need(proj.dtype == torch.float32 and proj.dim() == 2 and proj.stride(1) == 1 and proj.shape[1] == 2 * heads * dim + heads * vdim,
+          "proj must be float32 [T, %d] with unit inner stride, got %s %s", 2 * heads * dim + heads * vdim, proj.dtype, tuple(proj.shape))
+    _need(0 < dim <= HGRN2_MAX_DIM, "the recurrence kernel takes up to %d key channels per head, got %d", HGRN2_MAX_DIM, dim)
+    _f32(f_bias, (heads * dim,), "f_bias")
+    _f32(lower, (heads * dim,), "lower")
+    _need(state.dtype == torch.float32 and state.dim() == 4 and state.is_contiguous() and tuple(state.shape[1:]) == (heads, dim, vdim),
+          "state must be contiguous float32 [slots, %d, %d, %d]", heads, dim, vdim)
+    E = step.cu_tokens.shape[0] - 1
+    _need(slots.dtype == torch.int64 and slots.shape == (E,) and slots.is_contiguous(), "slots must be contiguous int64 [%d]", E)
+    _need(update, "the recurrence always advances its state")
+    out = torch.empty((T, heads, vdim), dtype=torch.float32, device=proj.device)
+    lib = build.load("gated_recurrence")
+    _check(lib.ga_hgrn2_scan(_ptr(out), _ptr(proj), _i64(proj.stride(0)), _ptr(f_bias), _ptr(lower), _ptr(state), _ptr(slots),
+                             _ptr(step.cu_tokens), _ptr(step.q_start), _i(E), _i(heads), _i(dim), _i(vdim), _stream()), "hgrn2_scan")
+    return out
+
+
+def headwise_rmsnorm(x, weight, eps, dtype):
+    """x float32 [..., V] -> the same shape in `dtype`: every row of V normalised by its root mean square, times weight [V]."""
+    _dev(x, weight)
+    _need(x.dtype == torch.float32 and x.is_contiguous(), "x must be contiguous float32")
+    V = x.shape[-1]
+    _f32(weight, (V,), "weight")
+    out = torch.empty(x.shape, dtype=dtype, device=x.device)
+    lib = build.load("gated_recurrence")
+    _check(lib.ga_headwise_rmsnorm(_ptr(out), _ptr(x), _ptr(weight), _i64(x.numel() // V), _i(V), _f(eps), _i(_is_bf16(dtype)),
+                                   _stream()), "headwise_rmsnorm")
+    return out
+
+
+LATENT_MAX_RANK = 512
+
+
+def latent_prepare(proj, q_norm, kv_norm, slot_mapping, c_pages, q_rank, kv_rank, heads, eps, dtype, write=True, gated=True):
+    """proj float32 [T, q_rank + kv_rank (+ heads)]: the down-projections (and gate logits).  Returns (cq [T, q_rank] in
+    `dtype`: the normed query latent; gate float32 [T, heads] or None); writes the normed latent c of every token into its
+    slot of c_pages [pages, page_size * kv_rank] (slot -1: no write)."""
+    _dev(proj, q_norm, kv_norm, slot_mapping, c_pages)
+    T = proj.shape[0]
+    cols = q_rank + kv_rank + (heads if gated else 0)
+    _need(proj.dtype == torch.float32 and proj.dim() == 2 and proj.stride(1) == 1 and proj.shape[1] == cols,
+          "proj must be float32 [T, %d], got %s %s", cols, proj.dtype, tuple(proj.shape))
+    _f32(q_norm, (q_rank,), "q_norm")
+    _f32(kv_norm, (kv_rank,), "kv_norm")
+    _need(slot_mapping.dtype == torch.int64 and slot_mapping.shape == (T,) and slot_mapping.is_contiguous(),
+          "slot_mapping must be contiguous int64 [T]")
+    _need(c_pages.dtype == dtype and c_pages.dim() == 2 and c_pages.is_contiguous() and c_pages.shape[1] % kv_rank == 0,
+          "the latent's pages must be contiguous %s [pages, page_size * %d]", dtype, kv_rank)
+    cq = torch.empty((T, q_rank), dtype=dtype, device=proj.device)
+    gate = torch.empty((T, heads), dtype=torch.float32, device=proj.device) if gated else None
+    lib = build.load("latent_attention")
+    _check(lib.ga_latent_prepare(_ptr(cq), _ptr(c_pages), _ptr(gate), _ptr(proj), _i64(proj.stride(0)), _ptr(q_norm), _ptr(kv_norm),
+                                 _ptr(slot_mapping), _i(T), _i(q_rank), _i(kv_rank), _i(heads), _f(eps), _i(1 if write else 0),
+                                 _i(_is_bf16(dtype)), _stream()), "latent_prepare")
+    return cq, gate
+
+
+def latent_attention(qa, c_pages, block_table, step, sink, gate, heads, rank, page_size, scale, window, dtype):
+    """qa float32 [heads, T, rank]: the queries in the latent space.  Every token attends to the latent rows of its request's
+    pages at positions [max(0, p - window + 1), p] (window None: from 0); sink float32 [heads] or None joins the softmax's
+    denominator; gate float32 [T, heads] or None scales each head's result.  Returns [heads, T, rank] in `dtype`."""
+    _dev(qa, c_pages, block_table, sink, gate)
+    T = step.token_entry.shape[0]
+    _f32(qa, (heads, T, rank), "qa")
+    _need(0 < rank <= LATENT_MAX_RANK, "the latent attention kernel takes ranks up to %d, got %d", LATENT_MAX_RANK, rank)
+    _need(c_pages.dtype == dtype and c_pages.dim() == 2 and c_pages.is_contiguous() and c_pages.shape[1] == page_size * rank,
+          "the latent's pages must be contiguous %s [pages, %d]", dtype, page_size * rank)
+    _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous(),
+          "block_table must be contiguous int32 [entries, width]")
+    for name, a in (("token_entry", step.token_entry), ("positions", step.positions)):
+        _need(a.dtype == torch.int32 and a.shape == (T,) and a.is_contiguous(), "%s must be contiguous int32 [T]", name)
+    if sink is not None:
+        _f32(sink, (heads,), "sink")
+    if gate is not None:
+        _f32(gate, (T, heads), "gate")
+    out = torch.empty((heads, T, rank), dtype=dtype, device=qa.device)
+    lib = build.load("latent_attention")
+    _check(lib.ga_latent_attention(_ptr(out), _i64(rank), _i64(T * rank), _ptr(qa), _i64(rank), _i64(T * rank), _ptr(c_pages),
+                                   _ptr(block_table), _i(block_table.shape[1]), _ptr(step.token_entry), _ptr(step.positions),
+                                   _ptr(sink), _ptr(gate), _i(T), _i(heads), _i(rank), _i(page_size), _i(int(window) if window else 0),
+                                   _f(scale), _i(_is_bf16(dtype)), _stream()), "latent_attention")
+    return out

@@ -13,6 +13,7 @@ class Arrangement:
     several parts that keep something returns the list of their specs and gets the list of views as `cache`)."""
 
     roles = {}
+    optional_roles = ()      # roles that a layer of this kind may leave out
 
     def __init__(self, parts):
         self._parts = dict(parts)
@@ -76,6 +77,50 @@ class PreNormBlock(Arrangement):
         if into_norm is not None:
             return self.feed_forward.forward(a, into_norm=(residual, into_norm))
         return self.feed_forward.forward(a)
+
+
+@register_arrangement("outnorm")
+class OutputNormBlock(Arrangement):
+    """x <- x + norm1(mixer(conv(x)));  x <- x + norm2(feed_forward(x)): the norms sit on the sublayers' OUTPUTS, and the
+    sublayers read the residual stream itself (the mixer through an optional short convolution over time).  A layer may
+    have no feed-forward (then it has no second norm either) and no convolution.  The norms are of a kind that offers
+    `add_normed(residual, y, copy)`.  The 32-bit stream is updated in place; nothing is left pending for the next block.
+    What a run keeps per request is the convolution's state followed by the mixer's cache, as a list."""
+
+    roles = {"mixer": "mixer", "mixer_norm": "norm", "feed_forward": "feed_forward", "feed_forward_norm": "norm",
+             "input_conv": "convolution"}
+    optional_roles = ("feed_forward", "feed_forward_norm", "input_conv")
+
+    def __init__(self, parts):
+        super().__init__(parts)
+        self.input_conv = self._parts.get("input_conv")
+        self.feed_forward = self._parts.get("feed_forward")
+        self.feed_forward_norm = self._parts.get("feed_forward_norm")
+        if (self.feed_forward is None) != (self.feed_forward_norm is None):
+            raise ValueError("a block names its feed-forward and that feed-forward's norm together, or neither")
+        for norm in (self.mixer_norm, self.feed_forward_norm):
+            if norm is not None and not hasattr(norm, "add_normed"):
+                raise ValueError("the norms of this block sit on the sublayers' outputs: %s has no add_normed"
+                                 % type(norm).__name__)
+
+    def cache_spec(self):
+        conv = self.input_conv.cache_spec() if self.input_conv is not None else None
+        return [conv, self.mixer.cache_spec()]
+
+    def forward(self, residual, delta, step, cache):
+        if delta is not None:                     # what a block of another kind left pending
+            residual.add_(whole(delta).to(residual.dtype))
+        conv_cache, mixer_cache = cache
+        dtype = self.mixer_norm.dtype
+        if self.input_conv is not None:
+            h = self.input_conv.forward(residual, step, conv_cache)
+        else:
+            h = residual if dtype == residual.dtype else residual.to(dtype)
+        m = self.mixer.forward(h, step, mixer_cache)
+        x = self.mixer_norm.add_normed(residual, m, copy=self.feed_forward is not None)
+        if self.feed_forward is not None:
+            self.feed_forward_norm.add_normed(residual, self.feed_forward.forward(x))
+        return None
 
 
 def whole(delta, norm=None):

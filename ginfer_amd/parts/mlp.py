@@ -44,3 +44,33 @@ class SwiGLU(Part):
                 return folded
         # the result may be partial sums of a K-split product: the norm that follows adds them up
         return linear(act, self.w_down, parts_ok=True)
+
+
+@register_feed_forward("clamped_glu")
+class ClampedGLU(Part):
+    """down(g * sigmoid(alpha g) * (u + shift)) with g = min(gate(x), limit) and u = clamp(up(x), -limit, limit); no
+    biases.  limit, alpha and shift are the model's constants.  Gate and up are one product over the stacked weights.
+    The tensors are named gate, up and down."""
+
+    capturable = True
+
+    def __init__(self, hidden_size, intermediate_size, limit, dtype, device, alpha=1.702, shift=1.0):
+        self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
+        self.limit, self.alpha, self.shift = float(limit), float(alpha), float(shift)
+        self.dtype, self.device = dtype, device
+        self.w_gate_up = self.w_down = None
+
+    def weight_specs(self):
+        H, I = self.hidden_size, self.intermediate_size
+        return {"gate": WeightSpec((I, H)), "up": WeightSpec((I, H)), "down": WeightSpec((H, I))}
+
+    def bind_weights(self, t):
+        self.w_gate_up = torch.cat([t["gate"], t["up"]], dim=0).contiguous()
+        self.w_down = t["down"]
+
+    def kernel_modules(self):
+        return ["activation", "gemm"] + (["gemm_skinny"] if self.dtype == torch.bfloat16 else [])
+
+    def forward(self, x):
+        act = ops.clamped_glu(linear(x, self.w_gate_up), self.limit, self.alpha, self.shift)
+        return linear(act, self.w_down)

@@ -74,10 +74,12 @@ class DecoderModel:
         for i, ls in enumerate(spec.layers):
             arrangement = registry.lookup("arrangement", ls.arrangement)
             roles = arrangement.roles        # role -> family of parts
-            if set(ls.parts) != set(roles):
-                raise ValueError("layer %d: arrangement %r has the roles %s, the layer names %s"
-                                 % (i, ls.arrangement, sorted(roles), sorted(ls.parts)))
-            self.blocks.append(arrangement({role: self._build(roles[role], ls.parts[role]) for role in roles}))
+            optional = set(getattr(arrangement, "optional_roles", ()))
+            if not (set(roles) - optional <= set(ls.parts) <= set(roles)):
+                raise ValueError("layer %d: arrangement %r has the roles %s (optional: %s), the layer names %s"
+                                 % (i, ls.arrangement, sorted(roles), sorted(optional), sorted(ls.parts)))
+            self.blocks.append(arrangement({role: self._build(roles[role], ls.parts[role]) for role in roles
+                                            if role in ls.parts}))
         self.schedule = list(spec.schedule)
         # per run of the schedule: the first norm of the block that runs next, where this run's block can fold it
         # into its own last product and that block takes its input so (a matter of speed only)
@@ -113,17 +115,17 @@ class DecoderModel:
         specs = {}
         for prefix, part in self._named_parts():
             for local, ws in part.weight_specs().items():
-                specs[prefix + "." + local] = ws
+                specs[_join(prefix, local)] = ws
         return specs
 
     def unread_weights(self):
         """Full names of tensors that a checkpoint may carry although no part reads them."""
-        return [prefix + "." + local for prefix, part in self._named_parts()
+        return [_join(prefix, local) for prefix, part in self._named_parts()
                 for local in getattr(part, "unread_weights", list)()]
 
     def bind_weights(self, tensors):
         for prefix, part in self._named_parts():
-            local = {n: tensors[prefix + "." + n] for n in part.weight_specs()}
+            local = {n: tensors[_join(prefix, n)] for n in part.weight_specs()}
             part.bind_weights(local)
         if getattr(self.head, "tied", False):
             self.head.tie(self.embedding.weight)
@@ -165,6 +167,12 @@ class DecoderModel:
                 delta = self.blocks[e.layer].forward(residual, delta, step, cache)
         n = self.final_norm.forward(residual, whole(delta, self.final_norm), rows=step.logit_rows)
         return self.head.forward(n)
+
+
+def _join(prefix, local):
+    """A tensor's full name: the part's prefix and the tensor's name inside the part; a part's tensor with an empty
+    name is called as the part itself."""
+    return prefix + "." + local if local else prefix
 
 
 def build_model(spec, dtype, device):

@@ -3,7 +3,7 @@ reaches it, so no part knows which model it is in.  New kinds register themselve
 decorators below; the model builder looks kinds up here and nowhere else."""
 
 _REGISTRIES = {"mixer": {}, "feed_forward": {}, "norm": {}, "position": {}, "embedding": {}, "head": {},
-               "arrangement": {}}
+               "arrangement": {}, "convolution": {}}
 
 
 def _register(role, kind):
@@ -35,6 +35,10 @@ def register_embedding(kind):
 
 def register_head(kind):
     return _register("head", kind)
+
+
+def register_convolution(kind):
+    return _register("convolution", kind)
 
 
 def register_arrangement(kind):

@@ -20,7 +20,7 @@ from .safetensors_file import open_model_files
 class WeightSpec:
     shape: Tuple[int, ...]
     kind: str = "float"          # "float" or "int"
-    init: str = "normal"         # "normal" N(0, std), "one_plus_normal" 1 + N(0, std), "zeros", "ones"
+    init: str = "normal"         # "normal" N(0, std), "one_plus_normal" 1 + N(0, std), "unit_interval" inside (0, 1), "zeros", "ones"
     std: float = 0.02
     keep_32bit: bool = False     # a tensor stored in 32-bit stays in 32-bit
 

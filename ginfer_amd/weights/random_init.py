@@ -22,6 +22,16 @@ def _tensor_seed(seed, name):
     return int.from_bytes(h[:8], "little") & ((1 << 63) - 1)
 
 
+# the mean of each kind of draw.  "unit_interval": numbers inside (0, 1), 0.5 + N(0, 0.2) cut off at bounds that every
+# storage dtype holds exactly (so cutting before or after the rounding gives the same), whatever std the spec names
+_MEANS = {"normal": 0.0, "one_plus_normal": 1.0, "unit_interval": 0.5}
+_UNIT_BOUNDS = (1.0 / 64.0, 63.0 / 64.0)
+
+
+def _std(spec, std_scale):
+    return 0.2 if spec.init == "unit_interval" else spec.std * std_scale
+
+
 def draw(spec, seed, name, dtype, std_scale=1.0):
     """One tensor on the host: element i is mean + std * normal(key of (seed, name), i) from the counter-based
     generator that the device kernel shares (csrc/random_normal.h), rounded once to `dtype`."""
@@ -31,7 +41,7 @@ def draw(spec, seed, name, dtype, std_scale=1.0):
         return torch.zeros(spec.shape, dtype=dtype)
     if spec.init == "ones":
         return torch.ones(spec.shape, dtype=dtype)
-    if spec.init not in ("normal", "one_plus_normal"):
+    if spec.init not in _MEANS:
         raise ValueError("unknown init %r for %s" % (spec.init, name))
     import ctypes
     from ..kernels import build
@@ -39,10 +49,12 @@ def draw(spec, seed, name, dtype, std_scale=1.0):
     t = torch.empty(spec.shape, dtype=torch.float32)
     rc = lib.ga_random_normal_fill_host(ctypes.c_void_p(t.data_ptr()), ctypes.c_int64(t.numel()),
                                         ctypes.c_uint64(_tensor_seed(seed, name)),
-                                        ctypes.c_float(1.0 if spec.init == "one_plus_normal" else 0.0),
-                                        ctypes.c_float(spec.std * std_scale), ctypes.c_int(min(16, os.cpu_count() or 1)))
+                                        ctypes.c_float(_MEANS[spec.init]),
+                                        ctypes.c_float(_std(spec, std_scale)), ctypes.c_int(min(16, os.cpu_count() or 1)))
     if rc != 0:
         raise RuntimeError("the host's random fill failed for %s (code %d)" % (name, rc))
+    if spec.init == "unit_interval":
+        t.clamp_(*_UNIT_BOUNDS)
     return t.to(dtype)
 
 
@@ -62,11 +74,12 @@ def bind_random_weights(model, seed, device, std_scale=1.0):
         dt = target_dtype(spec, model.dtype, model.dtype)       # as a checkpoint stored in the compute dtype would load
         if spec.init in ("zeros", "ones"):
             return torch.full(spec.shape, 0.0 if spec.init == "zeros" else 1.0, dtype=dt, device=device)
-        if spec.init not in ("normal", "one_plus_normal"):
+        if spec.init not in _MEANS:
             raise ValueError("unknown init %r for %s" % (spec.init, name))
         out = torch.empty(spec.shape, dtype=dt, device=device)
-        ops.random_normal_fill(out, _tensor_seed(seed, name), 1.0 if spec.init == "one_plus_normal" else 0.0,
-                               spec.std * std_scale)
+        ops.random_normal_fill(out, _tensor_seed(seed, name), _MEANS[spec.init], _std(spec, std_scale))
+        if spec.init == "unit_interval":
+            out.clamp_(*_UNIT_BOUNDS)
         return out
     tensors = TensorsOnDemand(specs, make)
     model.bind_weights(tensors)
