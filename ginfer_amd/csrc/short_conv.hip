@@ -23,7 +23,8 @@ __global__ __launch_bounds__(SC_THREADS) void short_conv_apply_kernel(T* __restr
   const int e = token_entry[t];
   const int local = (int)t - cu[e];                 // place of the token among the entry's tokens of this step
   const bool fresh = q_start[e] == 0;
-  const float* st = state + slots[e] * (int64_t)(taps - 1) * width;
+  // with one tap there is no state, and neither `state` nor `slots` is given
+  const float* st = taps > 1 ? state + slots[e] * (int64_t)(taps - 1) * width : nullptr;
   for (int c = blockIdx.y * SC_THREADS + threadIdx.x; c < width; c += gridDim.y * SC_THREADS) {
     float acc = add_input ? x[t * width + c] : 0.f;
     for (int j = 0; j < taps; ++j) {
@@ -66,7 +67,7 @@ extern "C" int ga_short_conv_apply(void* out, const void* x, const void* w, cons
                                    int taps, int add_input, int out_bf16, hipStream_t stream) {
   if (tokens <= 0) return 0;
   if (width <= 0 || taps < 1 || taps > SC_MAX_TAPS) return -1;
-  if (taps > 1 && state == nullptr) return -2;
+  if (taps > 1 && (state == nullptr || slots == nullptr)) return -2;
   int cols = (width + SC_THREADS - 1) / SC_THREADS;
   if (cols > 64) cols = 64;
   dim3 grid(tokens, cols), block(SC_THREADS);

@@ -31,7 +31,7 @@ class HGRN2(Part):
 
     def weight_specs(self):
         H, k, v = self.hidden_size, self.nh * self.dk, self.nh * self.dv
-        return {"q": WeightSpec((k, H)), "f": WeightSpec((k, H)), "f.b": WeightSpec((k,), std=1.0),
+        return {"q": WeightSpec((k, H)), "f": WeightSpec((k, H)), "f.b": WeightSpec((k,), std=0.2),
                 "lower": WeightSpec((k,), init="unit_interval"), "v": WeightSpec((v, H)),
                 "norm": WeightSpec((self.dv,), init="one_plus_normal"), "o": WeightSpec((H, v))}
 

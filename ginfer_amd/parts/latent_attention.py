@@ -34,7 +34,7 @@ class LatentAttention(Part):
         self.window = int(window) if window else None
         self.eps, self.dtype, self.device = float(eps), dtype, device
         self.has_sink, self.gated = bool(sink), bool(gated)
-        self.w_down = self.q_norm = self.kv_norm = self.w_uq = self.w_uk = self.w_uv_t = self.sink = self.w_o = None
+        self.w_down = self.q_norm = self.kv_norm = self.w_uq = self.w_uk_t = self.w_uv = self.sink = self.w_o = None
 
     def cache_spec(self):
         return PagedSpec((("c", self.kv_rank),), self.window)
@@ -47,7 +47,7 @@ class LatentAttention(Part):
                  "uk": WeightSpec((nh * self.hd, self.kv_rank)), "uv": WeightSpec((nh * self.vd, self.kv_rank)),
                  "o": WeightSpec((H, nh * self.vd))}
         if self.has_sink:
-            specs["sink"] = WeightSpec((nh,), std=1.0)
+            specs["sink"] = WeightSpec((nh,), std=0.2)
         if self.gated:
             specs["g"] = WeightSpec((nh, H))
         return specs
@@ -58,8 +58,8 @@ class LatentAttention(Part):
         self.q_norm = t["dq.norm"].float().contiguous()
         self.kv_norm = t["dkv.norm"].float().contiguous()
         self.w_uq = t["uq"]
-        self.w_uk = t["uk"].view(self.nh, self.hd, self.kv_rank).contiguous()                     # [head][dim][rank]
-        self.w_uv_t = t["uv"].view(self.nh, self.vd, self.kv_rank).transpose(1, 2).contiguous()   # [head][rank][vdim]
+        self.w_uk_t = t["uk"].view(self.nh, self.hd, self.kv_rank).transpose(1, 2).contiguous()   # [head][rank][dim]
+        self.w_uv = t["uv"].view(self.nh, self.vd, self.kv_rank).contiguous()                     # [head][vdim][rank]
         self.sink = t["sink"].float().contiguous() if self.has_sink else None
         self.w_o = t["o"]
 
@@ -73,13 +73,20 @@ class LatentAttention(Part):
         cq, gate = ops.latent_prepare(proj, self.q_norm, self.kv_norm, cache.slot_mapping, c_pages, self.q_rank,
                                       self.kv_rank, self.nh, self.eps, self.dtype, write=cache.owner, gated=self.gated)
         q = linear(cq, self.w_uq).view(T, self.nh, self.hd).transpose(0, 1)                       # [head][T][dim]
-        # the queries carried into the latent space, head by head, in 32-bit
+        # the queries carried into the latent space, head by head, in 32-bit.  bfloat16: one batched product of the
+        # library; float32: the package's own product per head, whose bits do not depend on the number of rows
         if self.dtype == torch.float32:
-            qa = torch.bmm(q, self.w_uk)
+            qa = torch.empty((self.nh, T, self.kv_rank), dtype=torch.float32, device=x.device)
+            for h in range(self.nh):
+                ops.gemm_nt(q[h], self.w_uk_t[h], out=qa[h])
         else:
-            qa = torch.bmm(q, self.w_uk, out_dtype=torch.float32)
+            qa = torch.bmm(q, self.w_uk_t.transpose(1, 2), out_dtype=torch.float32)
         a = ops.latent_attention(qa, c_pages, cache.block_table, step, self.sink, gate, self.nh, self.kv_rank,
                                  cache.page_size, self.scale, self.window, self.dtype)            # [head][T][rank]
         o = torch.empty((T, self.nh, self.vd), dtype=self.dtype, device=x.device)
-        torch.bmm(a, self.w_uv_t, out=o.transpose(0, 1))
+        if self.dtype == torch.float32:
+            for h in range(self.nh):
+                ops.gemm_nt(a[h], self.w_uv[h], out=o[:, h])
+        else:
+            torch.bmm(a, self.w_uv.transpose(1, 2), out=o.transpose(0, 1))
         return linear(o.view(T, self.nh * self.vd), self.w_o)
