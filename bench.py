@@ -55,6 +55,96 @@ def model_numbers(cfg, layers):
     return weight_bytes, kv_bytes_per_token, prefill_flops
 
 
+# Layer sizes for the Titozen design beside Qwen2 at equal width, feed-forward, layers and vocabulary (--titozen): two
+# recurrent layers to one of latent attention, as the design's small models have them.
+def _titozen_size(width, ff, heads, kv_rank, q_rank, window, kv_heads, layers=6, vocab=32768):
+    hg = dict(type="hgrn2", mixer=dict(heads=heads, dim=64, vdim=128), mlp=dict(kind="dense", ff=ff, limit=7.0))
+    la = dict(type="latent_attention", mlp=dict(kind="dense", ff=ff, limit=7.0),
+              mixer=dict(heads=heads, dim=128, vdim=128, q_rank=q_rank, kv_rank=kv_rank, scale=128 ** -0.5, mask=dict(size=window)))
+    titozen = dict(architecture="Titozen", vocab=vocab, width=width, norm=dict(eps=1e-5), canon=dict(taps=4),
+                   layers=[la if i % 3 == 2 else hg for i in range(layers)])
+    qwen2 = dict(SHAPE, num_hidden_layers=layers, hidden_size=width, num_attention_heads=heads, num_key_value_heads=kv_heads,
+                 head_dim=128, intermediate_size=ff, vocab_size=vocab, max_position_embeddings=32768)
+    return titozen, qwen2
+
+
+TITOZEN_SIZES = {"1.5b": _titozen_size(1536, 8960, 12, 256, 768, 1024, 2), "7b": _titozen_size(3584, 18944, 28, 512, 1536, 2048, 4)}
+
+
+def compare_titozen(args):
+    """Prefill of --prefill-tokens tokens and decode steps at --batch and the --points (contexts ending at --context)
+    through Engine.step, for each size and each of the two designs."""
+    import torch
+    from ginfer_amd import Engine, EngineConfig, SamplingParams, config_from_dict
+    page, T, C = 16, args.prefill_tokens, args.context
+    batches = sorted({int(p) for p in args.points.split(",") if p} | {args.batch})
+    max_b = max(batches)
+    g = torch.Generator().manual_seed(0)
+    out = {"metric": "prefill and decode tok/s of the Titozen design beside Qwen2 at equal sizes", "unit": "tok/s", "n_gpus": 1,
+           "steps": args.steps, "warmup": args.warmup, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+           "data": "synthetic tokens, random weights", "prefill_tokens": T, "context": C, "sizes": {}}
+    for size in [x for x in args.titozen.split(",") if x]:
+        if size not in TITOZEN_SIZES:
+            sys.exit("bench.py: --titozen takes %s, got %r" % (", ".join(sorted(TITOZEN_SIZES)), size))
+        row = {}
+        for design, cfg in zip(("titozen", "qwen2"), TITOZEN_SIZES[size]):
+            engine = Engine(EngineConfig(
+                model_path=None, model_config=config_from_dict(cfg), random_seed=0, dtype=args.dtype,
+                max_num_batched_tokens=max(2048, T, C) + max_b, max_num_seqs=max_b, max_seq_len=max(T, C) + max_b + 24,
+                kvcache_block_size=page, num_kvcache_blocks=max_b * -(-(C + 24) // page) + -(-T // page) + 8,
+                enable_prefix_caching=False, warmup=not args.no_engine_warmup))
+            vocab = engine.runner.vocab_size
+            res = {"weights_MB": round(sum(int(torch.tensor(ws.shape).prod()) for ws in engine.runner.model.weight_specs().values())
+                                       * (2 if args.dtype == "bfloat16" else 4) / 1e6, 1)}
+            times = []
+            for _ in range(4):
+                engine.add_request(torch.randint(0, vocab, (T,), generator=g).tolist(), SamplingParams(max_tokens=1, ignore_eos=True))
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                done = engine.step()
+                torch.cuda.synchronize()
+                times.append(time.perf_counter() - t0)
+                assert len(done) == 1 and not engine.has_unfinished()
+            res["prefill_tok_s"], res["prefill_ms"] = round(T / min(times[1:]), 1), round(min(times[1:]) * 1e3, 3)
+            for B in batches:
+                params = SamplingParams(max_tokens=args.steps + args.warmup + B + 16, ignore_eos=True)
+                engine.config.pipeline_decode = False
+                ids = []
+                for i in range(B):
+                    n = C - args.steps - args.warmup - (B - 1 - i)
+                    ids.append(engine.add_request(torch.randint(0, vocab, (n,), generator=g).tolist(), params))
+                    engine.step()
+                engine.config.pipeline_decode = True
+                for _ in range(args.warmup):
+                    engine.step()
+                torch.cuda.synchronize()
+                engine.step_log.clear()
+                t0 = time.perf_counter()
+                for _ in range(args.steps):
+                    engine.step()
+                torch.cuda.synchronize()
+                dt = (time.perf_counter() - t0) / args.steps
+                log = list(engine.step_log)
+                assert len(log) == args.steps and all(p == 0 and d == B for _, _, p, d in log), "a timed step was no decode step"
+                if not bool(torch.isfinite(engine.last_logits).all()):
+                    sys.exit("bench.py: the step that was just timed made logits that are not finite")
+                res["decode_b%d_tok_s" % B] = round(B / dt, 1)
+                res["decode_b%d_ms" % B] = round(dt * 1e3, 4)
+                res["decode_b%d_device_ms" % B] = round(1e3 * sum(d for _, d, _, _ in log) / args.steps, 4)
+                for rid in ids:
+                    engine.abort(rid)
+                while engine.has_unfinished():
+                    engine.step()
+            res["ran"] = dict(engine.runner.counts)
+            row[design] = res
+            del engine
+            import gc
+            gc.collect()
+            torch.cuda.empty_cache()
+        out["sizes"][size] = row
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -84,6 +174,10 @@ def main():
     ap.add_argument("--file-weights", action="store_true",
                     help="write the random weights into a model folder and load them from there, instead of drawing them "
                          "on the device (not for 72b: 145 GB)")
+    ap.add_argument("--titozen", default=None, metavar="SIZES",
+                    help="instead of the headline: prefill and decode throughput of the Titozen design at layer sizes that "
+                         "resemble real models (comma-separated: %s), each beside the Qwen2 design at equal width, "
+                         "feed-forward, layers and vocabulary; one JSON line" % ", ".join(sorted(TITOZEN_SIZES)))
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this engine runs on ONE GPU; --gpus %d is not supported" % args.gpus)
@@ -91,6 +185,10 @@ def main():
 
     import torch
     from ginfer_amd import Engine, EngineConfig, SamplingParams, config_from_dict, write_random_model
+
+    if args.titozen:
+        print(json.dumps(compare_titozen(args)))
+        return
 
     shape_name, shape = SHAPES[args.shape]
     full_layers = shape["num_hidden_layers"]
