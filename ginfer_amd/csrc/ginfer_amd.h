@@ -118,13 +118,31 @@ int ga_headwise_rmsnorm(void* out, const void* x, const void* weight, int64_t ro
 // (element strides per token and per head); window 0: all earlier keys; sink float [heads] or null; gate float
 // [tokens, heads] or null; out in the compute dtype (element strides per token and per head)
 int ga_latent_attention_max_rank();
-int ga_latent_prepare(void* cq, void* c_pages, void* gate, const void* proj, int64_t proj_stride, const void* wq,
-                      const void* wkv, const void* slot_mapping, int tokens, int q_rank, int kv_rank, int heads, float eps,
-                      int write_c, int is_bf16, hipStream_t stream);
+// ct_pages (or null): a second copy of the latent, transposed inside the page ([pages][rank][page_size])
+int ga_latent_prepare(void* cq, void* c_pages, void* ct_pages, int page_size, void* gate, const void* proj,
+                      int64_t proj_stride, const void* wq, const void* wkv, const void* slot_mapping, int tokens, int q_rank,
+                      int kv_rank, int heads, float eps, int write_c, int is_bf16, hipStream_t stream);
 int ga_latent_attention(void* out, int64_t out_t, int64_t out_h, const void* qa, int64_t qa_t, int64_t qa_h,
                         const void* c_pages, const void* block_table, int table_width, const void* token_entry,
                         const void* positions, const void* sink, const void* gate, int tokens, int heads, int rank,
                         int page_size, int window, float scale, int is_bf16, hipStream_t stream);
+
+// the same on the matrix cores, bfloat16, with both copies of the latent: rows = prompt portions, 16 neighbouring tokens as
+// columns (skip_singles: requests that bring one token are left to the other entry point; cu int32 [entries + 1]);
+// heads = single tokens, 16 heads as columns, info int32 [n][4] = (row, position, entry, -), the keys dealt to `splits`
+// workgroups of tiles_per_split tiles of 32 (ws_o: n * heads * splits * ga_latent_attention_mfma_padded_rank(rank)
+// floats, ws_ml: n * heads * splits * 2 floats; null for one split)
+int ga_latent_attention_mfma_padded_rank(int rank);
+int ga_latent_attention_rows(void* out, int64_t out_t, int64_t out_h, const void* qa, int64_t qa_t, int64_t qa_h,
+                             const void* c_pages, const void* ct_pages, const void* block_table, int table_width,
+                             const void* token_entry, const void* positions, const void* cu, const void* sink,
+                             const void* gate, int tokens, int heads, int rank, int page_size, int window, float scale,
+                             int skip_singles, hipStream_t stream);
+int ga_latent_attention_heads(void* out, int64_t out_t, int64_t out_h, void* ws_o, void* ws_ml, const void* qa, int64_t qa_t,
+                              int64_t qa_h, const void* c_pages, const void* ct_pages, const void* block_table,
+                              int table_width, const void* info, int n, const void* sink, const void* gate, int heads,
+                              int rank, int page_size, int window, float scale, int splits, int tiles_per_split,
+                              hipStream_t stream);
 
 // ---- attention_generic.hip: every token attends to its request's pages; any head size up to 256, window or 0;
 // tokens_per_workgroup neighbouring tokens share a workgroup's tiles of keys and values (0: the library chooses; -1: the

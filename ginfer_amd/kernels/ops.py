@@ -901,11 +901,13 @@ def headwise_rmsnorm(x, weight, eps, dtype):
 LATENT_MAX_RANK = 512
 
 
-def latent_prepare(proj, q_norm, kv_norm, slot_mapping, c_pages, q_rank, kv_rank, heads, eps, dtype, write=True, gated=True):
+def latent_prepare(proj, q_norm, kv_norm, slot_mapping, c_pages, q_rank, kv_rank, heads, eps, dtype, write=True, gated=True,
+                   ct_pages=None):
     """proj float32 [T, q_rank + kv_rank (+ heads)]: the down-projections (and gate logits).  Returns (cq [T, q_rank] in
     `dtype`: the normed query latent; gate float32 [T, heads] or None); writes the normed latent c of every token into its
-    slot of c_pages [pages, page_size * kv_rank] (slot -1: no write)."""
-    _dev(proj, q_norm, kv_norm, slot_mapping, c_pages)
+    slot of c_pages [pages, page_size * kv_rank] (slot -1: no write) and, where ct_pages is given, into the copy that
+    lies transposed inside each page ([pages, kv_rank * page_size])."""
+    _dev(proj, q_norm, kv_norm, slot_mapping, c_pages, ct_pages)
     T = proj.shape[0]
     cols = q_rank + kv_rank + (heads if gated else 0)
     _need(proj.dtype == torch.float32 and proj.dim() == 2 and proj.stride(1) == 1 and proj.shape[1] == cols,
@@ -914,22 +916,34 @@ def latent_prepare(proj, q_norm, kv_norm, slot_mapping, c_pages, q_rank, kv_rank
     _f32(kv_norm, (kv_rank,), "kv_norm")
     _need(slot_mapping.dtype == torch.int64 and slot_mapping.shape == (T,) and slot_mapping.is_contiguous(),
           "slot_mapping must be contiguous int64 [T]")
-    _need(c_pages.dtype == dtype and c_pages.dim() == 2 and c_pages.is_contiguous() and c_pages.shape[1] % kv_rank == 0,
-          "the latent's pages must be contiguous %s [pages, page_size * %d]", dtype, kv_rank)
+    for pages in (c_pages, ct_pages):
+        _need(pages is None or (pages.dtype == dtype and pages.dim() == 2 and pages.is_contiguous() and pages.shape[1] % kv_rank == 0
+                                and pages.shape == c_pages.shape),
+              "the latent's pages must be contiguous %s [pages, page_size * %d]", dtype, kv_rank)
     cq = torch.empty((T, q_rank), dtype=dtype, device=proj.device)
     gate = torch.empty((T, heads), dtype=torch.float32, device=proj.device) if gated else None
     lib = build.load("latent_attention")
-    _check(lib.ga_latent_prepare(_ptr(cq), _ptr(c_pages), _ptr(gate), _ptr(proj), _i64(proj.stride(0)), _ptr(q_norm), _ptr(kv_norm),
-                                 _ptr(slot_mapping), _i(T), _i(q_rank), _i(kv_rank), _i(heads), _f(eps), _i(1 if write else 0),
-                                 _i(_is_bf16(dtype)), _stream()), "latent_prepare")
+    _check(lib.ga_latent_prepare(_ptr(cq), _ptr(c_pages), _ptr(ct_pages), _i(c_pages.shape[1] // kv_rank), _ptr(gate), _ptr(proj),
+                                 _i64(proj.stride(0)), _ptr(q_norm), _ptr(kv_norm), _ptr(slot_mapping), _i(T), _i(q_rank),
+                                 _i(kv_rank), _i(heads), _f(eps), _i(1 if write else 0), _i(_is_bf16(dtype)), _stream()),
+           "latent_prepare")
     return cq, gate
 
 
-def latent_attention(qa, c_pages, block_table, step, sink, gate, heads, rank, page_size, scale, window, dtype):
+def latent_attention_mfma_supported(dtype, rank, page_size):
+    """The matrix-core kernels take bfloat16, ranks that are multiples of 8 up to 512 and page sizes that are powers of two
+    from 8."""
+    return dtype == torch.bfloat16 and rank % 8 == 0 and 0 < rank <= 512 and page_size >= 8 and page_size & (page_size - 1) == 0
+
+
+def latent_attention(qa, c_pages, block_table, step, sink, gate, heads, rank, page_size, scale, window, dtype, ct_pages=None):
     """qa float32 [heads, T, rank]: the queries in the latent space.  Every token attends to the latent rows of its request's
     pages at positions [max(0, p - window + 1), p] (window None: from 0); sink float32 [heads] or None joins the softmax's
-    denominator; gate float32 [T, heads] or None scales each head's result.  Returns [heads, T, rank] in `dtype`."""
-    _dev(qa, c_pages, block_table, sink, gate)
+    denominator; gate float32 [T, heads] or None scales each head's result.  Returns [heads, T, rank] in `dtype`.
+    With ct_pages (the copy transposed inside each page) and sizes that `latent_attention_mfma_supported` takes, the matrix
+    cores do it: prompt portions with 16 tokens side by side, single tokens with 16 heads side by side and their keys
+    dealt to several workgroups; else the general kernel."""
+    _dev(qa, c_pages, ct_pages, block_table, sink, gate)
     T = step.token_entry.shape[0]
     _f32(qa, (heads, T, rank), "qa")
     _need(0 < rank <= LATENT_MAX_RANK, "the latent attention kernel takes ranks up to %d, got %d", LATENT_MAX_RANK, rank)
@@ -945,8 +959,44 @@ def latent_attention(qa, c_pages, block_table, step, sink, gate, heads, rank, pa
         _f32(gate, (T, heads), "gate")
     out = torch.empty((heads, T, rank), dtype=dtype, device=qa.device)
     lib = build.load("latent_attention")
+    w = int(window) if window else 0
+    if ct_pages is not None and latent_attention_mfma_supported(dtype, rank, page_size):
+        _need(ct_pages.dtype == dtype and ct_pages.shape == c_pages.shape and ct_pages.is_contiguous(),
+              "the transposed copy must have the shape of the latent's pages")
+        info = (step.extra or {}).get("decode_info") if getattr(step, "extra", None) is not None else None
+        _need(info is not None and info.dtype == torch.int32 and info.dim() == 2 and info.shape[1] == 4 and info.is_contiguous(),
+              "the step must bring its single tokens as int32 [n, 4] (row, position, entry, 0)")
+        E = step.cu_tokens.shape[0] - 1
+        _need(step.cu_tokens.dtype == torch.int32 and step.cu_tokens.is_contiguous(), "cu_tokens must be contiguous int32")
+        n_single = info.shape[0]
+        if n_single < T:      # the step holds prompt portions (in a recorded step of padded sizes: may hold)
+            _check(lib.ga_latent_attention_rows(
+                _ptr(out), _i64(rank), _i64(T * rank), _ptr(qa), _i64(rank), _i64(T * rank), _ptr(c_pages), _ptr(ct_pages),
+                _ptr(block_table), _i(block_table.shape[1]), _ptr(step.token_entry), _ptr(step.positions), _ptr(step.cu_tokens),
+                _ptr(sink), _ptr(gate), _i(T), _i(heads), _i(rank), _i(page_size), _i(w), _f(scale), _i(1), _stream()),
+                "latent_attention_rows")
+        if n_single > 0:
+            # the longest walk in tiles of 32: over the window, or over the longest context of the step's bucket
+            span = int(step.extra.get("decode_span") or step.max_kv_len)
+            if w:
+                span = min(span, w)
+            tiles = (span + 31) // 32 + 1
+            workgroups = n_single * (-(-(-(-heads // 16)) // 4))
+            splits = max(1, min(tiles, TUNING.latent_decode_workgroups // max(workgroups, 1), TUNING.latent_decode_max_splits))
+            per = -(-tiles // splits)
+            splits = -(-tiles // per)
+            ws_o = ws_ml = None
+            if splits > 1:
+                rp = lib.ga_latent_attention_mfma_padded_rank(_i(rank))
+                ws_o = torch.empty((n_single * heads * splits * rp,), dtype=torch.float32, device=qa.device)
+                ws_ml = torch.empty((n_single * heads * splits * 2,), dtype=torch.float32, device=qa.device)
+            _check(lib.ga_latent_attention_heads(
+                _ptr(out), _i64(rank), _i64(T * rank), _ptr(ws_o), _ptr(ws_ml), _ptr(qa), _i64(rank), _i64(T * rank), _ptr(c_pages),
+                _ptr(ct_pages), _ptr(block_table), _i(block_table.shape[1]), _ptr(info), _i(n_single), _ptr(sink), _ptr(gate),
+                _i(heads), _i(rank), _i(page_size), _i(w), _f(scale), _i(splits), _i(per), _stream()), "latent_attention_heads")
+        return out
     _check(lib.ga_latent_attention(_ptr(out), _i64(rank), _i64(T * rank), _ptr(qa), _i64(rank), _i64(T * rank), _ptr(c_pages),
                                    _ptr(block_table), _i(block_table.shape[1]), _ptr(step.token_entry), _ptr(step.positions),
-                                   _ptr(sink), _ptr(gate), _i(T), _i(heads), _i(rank), _i(page_size), _i(int(window) if window else 0),
+                                   _ptr(sink), _ptr(gate), _i(T), _i(heads), _i(rank), _i(page_size), _i(w),
                                    _f(scale), _i(_is_bf16(dtype)), _stream()), "latent_attention")
     return out

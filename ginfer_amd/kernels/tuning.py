@@ -115,6 +115,11 @@ class Tuning:
     # to a workgroup as still leave `generic_fill_workgroups` workgroups (one and a half to a compute unit).
     generic_few_tokens_workgroups: int = 512
     generic_fill_workgroups: int = 384
+    # ---- the latent attention's matrix-core kernel for single tokens (csrc/latent_attention.hip): a token's keys are dealt
+    # to as many workgroups as bring the launch to about `latent_decode_workgroups` (four to a compute unit: a
+    # workgroup of it streams from memory no faster than any other), at most `latent_decode_max_splits` to a token
+    latent_decode_workgroups: int = 1024
+    latent_decode_max_splits: int = 32
     # ---- recorded steps (engine/runner.py): steps with prompt portions are laid into recorded steps of padded sizes up
     # to `mixed_graph_max_tokens` rows, fewer for large models: padding pays while rows x weights stays under what the
     # device does in the time the host needs to launch a step kernel by kernel.

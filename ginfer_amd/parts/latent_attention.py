@@ -37,6 +37,11 @@ class LatentAttention(Part):
         self.w_down = self.q_norm = self.kv_norm = self.w_uq = self.w_uk_t = self.w_uv = self.sink = self.w_o = None
 
     def cache_spec(self):
+        """The latent per token, in pages.  Where the matrix-core kernel can run (bfloat16, a rank in steps of 8) a page holds
+        a second copy, transposed ([rank][slot]): that kernel reads the latent as keys from the first and as values from
+        the second, each in 16-byte operands."""
+        if self.dtype == torch.bfloat16 and self.kv_rank % 8 == 0:
+            return PagedSpec((("c", self.kv_rank), ("ct", self.kv_rank)), self.window)
         return PagedSpec((("c", self.kv_rank),), self.window)
 
     def weight_specs(self):
@@ -69,9 +74,10 @@ class LatentAttention(Part):
     def forward(self, x, step, cache):
         T = x.shape[0]
         proj = linear(x, self.w_down, None, out_dtype=torch.float32)
-        c_pages = cache.pages["c"]
+        c_pages, ct_pages = cache.pages["c"], cache.pages.get("ct")
         cq, gate = ops.latent_prepare(proj, self.q_norm, self.kv_norm, cache.slot_mapping, c_pages, self.q_rank,
-                                      self.kv_rank, self.nh, self.eps, self.dtype, write=cache.owner, gated=self.gated)
+                                      self.kv_rank, self.nh, self.eps, self.dtype, write=cache.owner, gated=self.gated,
+                                      ct_pages=ct_pages)
         q = linear(cq, self.w_uq).view(T, self.nh, self.hd).transpose(0, 1)                       # [head][T][dim]
         # the queries carried into the latent space, head by head, in 32-bit.  bfloat16: one batched product of the
         # library; float32: the package's own product per head, whose bits do not depend on the number of rows
@@ -82,7 +88,7 @@ class LatentAttention(Part):
         else:
             qa = torch.bmm(q, self.w_uk_t.transpose(1, 2), out_dtype=torch.float32)
         a = ops.latent_attention(qa, c_pages, cache.block_table, step, self.sink, gate, self.nh, self.kv_rank,
-                                 cache.page_size, self.scale, self.window, self.dtype)            # [head][T][rank]
+                                 cache.page_size, self.scale, self.window, self.dtype, ct_pages=ct_pages)   # [head][T][rank]
         o = torch.empty((T, self.nh, self.vd), dtype=self.dtype, device=x.device)
         if self.dtype == torch.float32:
             for h in range(self.nh):

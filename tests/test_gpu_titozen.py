@@ -285,6 +285,87 @@ def test_latent_attention_sees_exactly_its_window(rank, heads, window, page):
                 assert err < 2e-5, "mark %s, sink %s, token %d: %.3g" % (mark, sink_value, i, err)
 
 
+@pytest.mark.parametrize("rank,heads,window,page", [(64, 6, 72, 16), (48, 3, 19, 8), (128, 20, 33, 16), (256, 5, 100, 32),
+                                                    (512, 17, None, 16), (136, 2, 40, 64)])
+def test_latent_attention_on_the_matrix_cores(rank, heads, window, page):
+    """bfloat16, both copies of the latent in the pages.  Three requests in one step: a portion of 21 tokens behind 140
+    cached ones, a single token behind 90, and a request's first 5 tokens (so a group of 16 neighbouring tokens holds two
+    requests); then a step of single tokens only, with the keys of each dealt to several workgroups.  In each, one row
+    just inside or just outside a window, or a far one, matches a query twenty times as well as the others."""
+    from ginfer_amd.kernels import ops
+    from ginfer_amd.kernels.tuning import TUNING
+    g = torch.Generator().manual_seed(rank + heads)
+    lens = [161, 91, 5]                              # cached + new tokens of the three requests
+    new = [21, 1, 5]
+    w = window or 10 ** 6
+    per_req = [-(-n // page) for n in lens]
+    order = torch.randperm(sum(per_req) + 2, generator=g)
+    width = max(per_req)
+    table = torch.full((3, width), -1, dtype=torch.int32)
+    rows, o = [], 0
+    for i, n in enumerate(lens):
+        table[i, :per_req[i]] = order[o:o + per_req[i]].int()
+        o += per_req[i]
+        rows.append((torch.randn((n, rank), generator=g) * 0.3).to(torch.bfloat16))
+    T = sum(new)
+    qa = torch.randn((heads, T, rank), generator=g)
+    # request 0: the last token's query finds the row just outside its window, the one before it the row just inside its own
+    last0 = new[0] - 1
+    for tok, key in ((last0, lens[0] - 1 - w), (last0 - 1, lens[0] - 2 - w + 1), (last0 - 2, 3), (new[0], lens[1] - 1 - w + 1)):
+        if 0 <= key:
+            req = 0 if tok <= last0 else 1
+            rows[req][key] = (qa[0, tok] / qa[0, tok].norm() * 20.0).to(torch.bfloat16)
+    pool = torch.zeros((sum(per_req) + 2, page * rank), dtype=torch.bfloat16)
+    pool_t = torch.zeros_like(pool)
+    for i, n in enumerate(lens):
+        for b in range(per_req[i]):
+            blk = rows[i][b * page:(b + 1) * page]
+            full = torch.zeros((page, rank), dtype=torch.bfloat16)
+            full[:blk.shape[0]] = blk
+            pool[table[i, b]] = full.reshape(-1)
+            pool_t[table[i, b]] = full.t().contiguous().reshape(-1)
+    gate = torch.rand((T, heads), generator=g)
+    sink = torch.randn((heads,), generator=g)
+
+    def reference(step_new, which):
+        out = torch.zeros((heads, sum(step_new), rank), dtype=torch.float64)
+        t = 0
+        for i, n in zip(which, step_new):
+            for k in range(n):
+                p = lens[i] - n + k
+                lo = max(0, p - w + 1)
+                c = rows[i][lo:p + 1].double()
+                q = qa_step[:, t].to(torch.bfloat16).double()
+                s = torch.einsum("hr,jr->hj", q, c) * 0.37
+                top = torch.maximum(s.max(dim=1).values, sink.double())
+                e = torch.exp(s - top[:, None])
+                den = e.sum(dim=1) + torch.exp(sink.double() - top)
+                out[:, t] = torch.einsum("hj,jr->hr", e / den[:, None], c) * gate_step[t].double()[:, None]
+                t += 1
+        return out
+
+    for step_new, which in ((new, [0, 1, 2]), ([1, 1], [0, 1])):
+        Ts = sum(step_new)
+        qa_step, gate_step = qa[:, :Ts].contiguous(), gate[:Ts].contiguous()
+        step = _Step(step_new, [lens[i] - n for i, n in zip(which, step_new)])
+        singles = [(int(step.cu_tokens[j]), lens[i] - 1, j, 0) for j, (i, n) in enumerate(zip(which, step_new)) if n == 1]
+        step.extra = {"decode_info": torch.tensor(singles, dtype=torch.int32).reshape(-1, 4).cuda(), "decode_span": 256}
+        step.max_kv_len = max(lens)
+        tbl = table[which].contiguous().cuda()
+        for splits in (1, 32):
+            old = TUNING.latent_decode_max_splits
+            TUNING.latent_decode_max_splits = splits
+            try:
+                got = ops.latent_attention(qa_step.cuda(), pool.cuda(), tbl, step, sink.cuda(), gate_step.cuda(), heads, rank, page,
+                                           0.37, window, torch.bfloat16, ct_pages=pool_t.cuda()).float().cpu()
+            finally:
+                TUNING.latent_decode_max_splits = old
+            ref = reference(step_new, which)
+            for t in range(Ts):
+                err = float((got[:, t].double() - ref[:, t]).abs().max() / max(float(ref[:, t].abs().max()), 1e-2))
+                assert err < 3e-2, "step %s, splits %d, token %d: %.3g" % (step_new, splits, t, err)
+
+
 def test_bounded_gated_activation():
     from ginfer_amd.kernels import ops
     g = torch.Generator().manual_seed(3)

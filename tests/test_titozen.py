@@ -62,7 +62,13 @@ def test_tensor_names_shapes_and_caches():
     assert "l1.norm2" not in shapes and "l1.mlp.gate" not in shapes and "l2.norm2" not in shapes
     specs = model.cache_specs()
     assert specs[0] == [StateSpec((2, 40)), StateSpec((2, 12, 20))]
-    assert specs[1] == [StateSpec((2, 40)), PagedSpec((("c", 10),), 21)]
+    assert specs[1] == [StateSpec((2, 40)), PagedSpec((("c", 10),), 21)]          # 32-bit: the latent alone
+    half = build_model(config_from_dict(CFG).model_spec(), torch.bfloat16, None).cache_specs()
+    assert half[1][1] == PagedSpec((("c", 10),), 21)                              # a rank that is no multiple of 8
+    c = copy.deepcopy(CFG)
+    c["layers"][1]["mixer"]["kv_rank"] = 16
+    half = build_model(config_from_dict(c).model_spec(), torch.bfloat16, None).cache_specs()
+    assert half[1][1] == PagedSpec((("c", 16), ("ct", 16)), 21)                   # bfloat16: and its transposed copy
     assert model.capturable()
 
 
