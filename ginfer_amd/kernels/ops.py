@@ -982,7 +982,7 @@ def latent_attention(qa, c_pages, block_table, step, sink, gate, heads, rank, pa
                 span = min(span, w)
             tiles = (span + 31) // 32 + 1
             workgroups = n_single * (-(-(-(-heads // 16)) // 4))
-            splits = max(1, min(tiles, TUNING.latent_decode_workgroups // max(workgroups, 1), TUNING.latent_decode_max_splits))
+            splits = max(1, min(tiles, TUNING.latent_decode_workgroups // max(workgroups, 1), TUNING.latent_decode_max_splits, 64))
             per = -(-tiles // splits)
             splits = -(-tiles // per)
             ws_o = ws_ml = None
