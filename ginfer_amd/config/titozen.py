@@ -27,7 +27,7 @@ LAYER_TENSOR_NAMES = dict(mixer="mix", feed_forward="mlp", mixer_norm="norm1", f
 MODEL_TENSOR_NAMES = dict(embedding="embed", final_norm="final.norm", head="head")
 
 _MIXER_KEYS = {"hgrn2": ("heads", "dim", "vdim"),
-               "latent_attention": ("heads", "dim", "vdim", "q_rank", "kv_rank", "scale", "mask")}
+               "latent_attention": ("heads", "dim", "vdim", "q_rank", "kv_rank", "scale")}
 
 
 def _int(d, key, where, minimum=1):
@@ -85,7 +85,7 @@ class TitozenConfig:
             if kind == "latent_attention":
                 mixer.update(q_rank=_int(m, "q_rank", where + " mixer"), kv_rank=_int(m, "kv_rank", where + " mixer"),
                              scale=_number(m, "scale", where + " mixer"))
-                mask = m["mask"]
+                mask = m.get("mask")             # no mask (or null): every earlier position is seen
                 mixer["mask"] = None if mask is None else dict(size=_int(mask, "size", where + " mixer mask"))
             mlp = l.get("mlp")
             if mlp is not None:

@@ -171,13 +171,24 @@ struct KRange {
 // are rows n0.. of the gate and the same rows of the up matrix, and the epilogue writes
 // silu(gate) * up = (g * (1 / (1 + exp(-g)))) * u (ginfer/core/op/kernels/cuda/swiglu_kernel.cu:24-27) for N
 // columns: the activation of the feed-forward without a pass over memory of its own.
+// The gate of a gated product: out = g * sigmoid(alpha g) * (u + shift) with g = min(gate, limit) and u = clamp(up, -limit,
+// limit).  limit = infinity, alpha = 1, shift = 0 is SiLU(gate) * up, bit for bit what stood here before the bounds.
+struct GateAct {
+  float limit, alpha, shift;
+};
+__device__ __forceinline__ float gate_act(float v, float u, const GateAct act) {
+  v = fminf(v, act.limit);
+  u = fminf(fmaxf(u, -act.limit), act.limit);
+  return (v * (1.0f / (1.0f + expf(-(act.alpha * v))))) * (u + act.shift);
+}
+
 template <int NT, int MB, int KS, typename TC, bool GATED, int PACK>
 __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(TC* __restrict__ C, int64_t ldc,
                                                                  const bf16_t* __restrict__ A, int64_t lda,
                                                                  const bf16_t* __restrict__ W,
                                                                  const bf16_t* __restrict__ bias, int M, int N,
                                                                  int K, int ksteps, NormIn norm_in,
-                                                                 NormOut norm_out, int fold_cols) {
+                                                                 NormOut norm_out, int fold_cols, GateAct act) {
   static_assert(PACK == 1 || MB == 1, "a packed tile holds at most 8 rows of A");
   __shared__ float red[SK_WAVES][NT * 16][MB * 16 + 1];
   __shared__ float rstd[16];
@@ -283,7 +294,7 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(TC* __restrict_
     if (GATED) {
       float u = total(gi, 1, nl, m);
       if (scale_rows) u *= rstd[m];
-      v = (v * (1.0f / (1.0f + expf(-v)))) * u;
+      v = gate_act(v, u, act);
     }
     if (bias && blockIdx.y == 0) v += bf16_to_f32(bias[n]);
     if (partial) Pp[(int64_t)m * N + n] = v;
@@ -306,7 +317,7 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_even_kernel(TC* __restrict__ 
                                                                const bf16_t* __restrict__ A, int64_t lda,
                                                                const bf16_t* __restrict__ W,
                                                                const bf16_t* __restrict__ bias, int M, int N, int K,
-                                                               int ksteps, NormIn norm_in) {
+                                                               int ksteps, NormIn norm_in, GateAct act) {
   static_assert(!GATED || TILES % 2 == 0, "as many tiles of the gate as of the up matrix");
   constexpr int PER = GATED ? TILES / 2 : TILES;             // tiles of one matrix
   __shared__ float red[SK_WAVES][TILES * 16][16 + 1];
@@ -352,7 +363,7 @@ __global__ __launch_bounds__(SK_THREADS) void gemm_even_kernel(TC* __restrict__ 
 #pragma unroll
       for (int w = 0; w < SK_WAVES; ++w) u += red[w][PER * 16 + cl][m];
       if (scale_rows) u *= rstd[m];
-      v = (v * (1.0f / (1.0f + expf(-v)))) * u;
+      v = gate_act(v, u, act);
     } else if (bias) {
       v += bf16_to_f32(bias[c0 + cl]);
     }
@@ -426,9 +437,9 @@ extern "C" int ga_skinny_norm_parts(int M, int N) {
 // by the consumer.  gated: W is [2N, K] (gate over up), C [M, N] = silu(A.gate^T) * (A.up^T), no bias, no
 // grid split.  M <= 64, K a multiple of 8, rows 16-byte aligned.  nt in {1,2,4}, ks in {1,2,4,8}, pack in
 // {1,2} (2: at most 8 rows); 0 lets the library choose.
-extern "C" int ga_gemm_skinny(void* C, int64_t ldc, const void* A, int64_t lda, const void* W, const void* bias,
+static int gemm_skinny_launch(void* C, int64_t ldc, const void* A, int64_t lda, const void* W, const void* bias,
                               int M, int N, int K, int out_f32, int nt, int ks, int grid_splits, int gated, int pack,
-                              const GaSkinnyNorm* norm, hipStream_t stream) {
+                              const GaSkinnyNorm* norm, GateAct act, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (M > 64 || K <= 0 || K % 8 || lda % 8 || grid_splits < 1) return -1;
   const int mb = (M + 15) / 16;
@@ -465,7 +476,7 @@ extern "C" int ga_gemm_skinny(void* C, int64_t ldc, const void* A, int64_t lda, 
     dim3 grid(workgroups), block(SK_THREADS);
 #define LAUNCH_EVEN(TILES, TC, G)                                                                              \
   hipLaunchKernelGGL((gemm_even_kernel<TILES, TC, G>), grid, block, 0, stream, (TC*)C, ldc, (const bf16_t*)A, \
-                     lda, (const bf16_t*)W, (const bf16_t*)bias, M, N, K, ksteps, norm_in)
+                     lda, (const bf16_t*)W, (const bf16_t*)bias, M, N, K, ksteps, norm_in, act)
 #define PICK_EVEN(TC)                                                                                          \
   if (gated) {                                                                                                 \
     if (per == 1) LAUNCH_EVEN(2, TC, true); else if (per == 2) LAUNCH_EVEN(4, TC, true); else LAUNCH_EVEN(6, TC, true); \
@@ -489,7 +500,7 @@ extern "C" int ga_gemm_skinny(void* C, int64_t ldc, const void* A, int64_t lda, 
 #define LAUNCH(NT, MB, KS, TC, G, PK)                                                                     \
   hipLaunchKernelGGL((gemm_skinny_kernel<NT, MB, KS, TC, G, PK>), grid, block, 0, stream, (TC*)C, ldc,   \
                      (const bf16_t*)A, lda, (const bf16_t*)W, (const bf16_t*)bias, M, N, K, ksteps,      \
-                     norm_in, norm_out, fcols)
+                     norm_in, norm_out, fcols, act)
 #define PICK_KS(NT, MB, TC, G, PK)                                                                        \
   switch (ks) {                                                                                           \
     case 1: LAUNCH(NT, MB, 1, TC, G, PK); break;                                                          \
@@ -524,6 +535,23 @@ extern "C" int ga_gemm_skinny(void* C, int64_t ldc, const void* A, int64_t lda, 
 #undef PICK_KS
 #undef LAUNCH
   return GA_CHECK_LAUNCH();
+}
+
+extern "C" int ga_gemm_skinny(void* C, int64_t ldc, const void* A, int64_t lda, const void* W, const void* bias,
+                              int M, int N, int K, int out_f32, int nt, int ks, int grid_splits, int gated, int pack,
+                              const GaSkinnyNorm* norm, hipStream_t stream) {
+  return gemm_skinny_launch(C, ldc, A, lda, W, bias, M, N, K, out_f32, nt, ks, grid_splits, gated, pack, norm,
+                            GateAct{INFINITY, 1.0f, 0.0f}, stream);
+}
+
+// The gated product with a bounded gate: C = g * sigmoid(alpha g) * (u + shift), g = min(A.gate^T, limit), u = clamp(A.up^T,
+// -limit, limit); everything else as ga_gemm_skinny with gated = 1.
+extern "C" int ga_gemm_skinny_bounded_gate(void* C, int64_t ldc, const void* A, int64_t lda, const void* W, int M, int N,
+                                           int K, int out_f32, int ks, int pack, float limit, float alpha, float shift,
+                                           const GaSkinnyNorm* norm, hipStream_t stream) {
+  if (!(limit > 0.f)) return -1;
+  return gemm_skinny_launch(C, ldc, A, lda, W, nullptr, M, N, K, out_f32, 2, ks, 1, 1, pack, norm, GateAct{limit, alpha, shift},
+                            stream);
 }
 
 // The fused q|k|v projection of a decode step with its epilogue: bias, NeoX rotation of q and k

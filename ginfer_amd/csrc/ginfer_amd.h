@@ -65,6 +65,11 @@ int ga_skinny_norm_parts(int M, int N);
 int ga_gemm_skinny(void* C, int64_t ldc, const void* A, int64_t lda, const void* W, const void* bias, int M, int N, int K,
                    int out_f32, int nt, int ks, int grid_splits, int gated, int pack, const struct GaSkinnyNorm* norm,
                    hipStream_t stream);
+// the gated product (W [2N, K], gate over up) with a bounded gate: C = g * sigmoid(alpha g) * (u + shift), g = min(gate, limit),
+// u = clamp(up, -limit, limit)
+int ga_gemm_skinny_bounded_gate(void* C, int64_t ldc, const void* A, int64_t lda, const void* W, int M, int N, int K,
+                                int out_f32, int ks, int pack, float limit, float alpha, float shift,
+                                const struct GaSkinnyNorm* norm, hipStream_t stream);
 int ga_qkv_rope_skinny(void* q_out, const void* A, int64_t lda, const void* W, const void* bias, const void* positions,
                        const void* cos_t, const void* sin_t, const void* slot_mapping, void* k_pages, void* v_pages,
                        int M, int K, int nh, int nkv, int hd, int page_size, int write_kv, int pack,

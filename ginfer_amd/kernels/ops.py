@@ -402,11 +402,12 @@ def gemm_skinny_supported(a, w):
 
 
 def gemm_skinny(a, w, bias=None, out=None, out_dtype=None, nt=0, ks=0, grid_splits=1, gated=False, into_norm=None,
-                pack=0):
+                pack=0, gate_bounds=None):
     """a [M <= 64, K] . w [N, K]^T (+ bias) -> [M, N] in bfloat16 (or float32): the decode step's products,
     weights streamed once through the matrix cores.  grid_splits > 1: K is split over workgroups too and
     the result is float32 [grid_splits, M, N], parts for the consumer to add.  gated: w is [2N, K] (gate
-    over up) and the result is silu(a.gate^T) * (a.up^T).
+    over up) and the result is silu(a.gate^T) * (a.up^T); with gate_bounds = (limit, alpha, shift) it is
+    g * sigmoid(alpha g) * (u + shift) with g = min(a.gate^T, limit) and u = clamp(a.up^T, -limit, limit).
     pack = 2 (at most 8 rows): a tile of the matrix cores holds 8 rows of w twice, for the two halves of K,
     so that twice the workgroups stream the weights.
     a may be ScaledRows (at most 16 rows): the rows of a norm in two factors.  into_norm = (residual, gain, eps):
@@ -465,6 +466,14 @@ def gemm_skinny(a, w, bias=None, out=None, out_dtype=None, nt=0, ks=0, grid_spli
         _need(out.shape == (M, N) and out.dtype == out_dtype and out.stride(1) == 1, "gemm_skinny: out must be [M, N]")
         ldc = out.stride(0)
     lib = build.load("gemm_skinny")
+    if gate_bounds is not None:
+        _need(gated and float(gate_bounds[0]) > 0, "gate bounds belong to a gated product, and the limit is positive")
+        limit, alpha, shift = gate_bounds
+        _check(lib.ga_gemm_skinny_bounded_gate(_ptr(out), _i64(ldc), _ptr(a), _i64(a.stride(0)), _ptr(w), _i(M), _i(N), _i(K),
+                                               _i(1 if out_dtype == torch.float32 else 0), _i(ks), _i(pack), _f(limit), _f(alpha),
+                                               _f(shift), ctypes.byref(norm) if norm is not None else _vp(0), _stream()),
+               "gemm_skinny_bounded_gate")
+        return out
     _check(lib.ga_gemm_skinny(_ptr(out), _i64(ldc), _ptr(a), _i64(a.stride(0)), _ptr(w), _ptr(bias), _i(M), _i(N),
                               _i(K), _i(1 if out_dtype == torch.float32 else 0), _i(nt), _i(ks), _i(grid_splits),
                               _i(1 if gated else 0), _i(pack), ctypes.byref(norm) if norm is not None else _vp(0),

@@ -4,7 +4,7 @@ import torch
 from ..kernels import ops
 from ..weights.loader import WeightSpec
 from .base import Part
-from .linear import linear, gated_linear, linear_into_norm
+from .linear import linear, gated_linear, gated_plan, linear_into_norm
 from .registry import register_feed_forward
 
 
@@ -72,5 +72,11 @@ class ClampedGLU(Part):
         return ["activation", "gemm"] + (["gemm_skinny"] if self.dtype == torch.bfloat16 else [])
 
     def forward(self, x):
-        act = ops.clamped_glu(linear(x, self.w_gate_up), self.limit, self.alpha, self.shift)
+        # few rows (decode): the weight-streaming product with the activation in its epilogue, where the rules would
+        # take that kernel for the SiLU gate too; else the product and the activation's own pass
+        if (x.dtype == torch.bfloat16 and ops.gemm_skinny_supported(x, self.w_gate_up)
+                and gated_plan(x.shape[0], self.w_gate_up.shape[0], True, False) == ("skinny",)):
+            act = ops.gemm_skinny(x, self.w_gate_up, gated=True, gate_bounds=(self.limit, self.alpha, self.shift))
+        else:
+            act = ops.clamped_glu(linear(x, self.w_gate_up), self.limit, self.alpha, self.shift)
         return linear(act, self.w_down)

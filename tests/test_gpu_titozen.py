@@ -137,7 +137,7 @@ class _Step:
 def test_norm_with_one_gain():
     from ginfer_amd.kernels import ops
     g = torch.Generator().manual_seed(0)
-    for H_ in (7, 96, 320, 1000):
+    for H_ in (7, 96, 328, 1000):
         x = torch.randn((5, H_), generator=g) * 3
         y = torch.randn((5, H_), generator=g)
         gain = torch.tensor([0.7])
@@ -198,7 +198,7 @@ def test_short_convolution_across_cuts_and_slots(taps):
             at[k] += n
 
 
-@pytest.mark.parametrize("heads,dim,vdim", [(1, 5, 3), (3, 48, 64), (2, 130, 20), (2, 16, 100), (1, 256, 16)])
+@pytest.mark.parametrize("heads,dim,vdim", [(1, 5, 3), (3, 40, 72), (2, 130, 20), (2, 16, 100), (1, 256, 16)])
 def test_gated_recurrence_across_cuts(heads, dim, vdim):
     """The recurrence of one request in portions of 1 to 40 tokens beside another request, against the plain loop; the
     forget gates reach from 0.02 to 0.98, so both what fades at once and what stays for the whole sequence count."""
@@ -241,7 +241,7 @@ def test_gated_recurrence_across_cuts(heads, dim, vdim):
     assert H.rel_err(got, pt.rms(refs["a"], 1e-5) * w.double()) < 1e-6
 
 
-@pytest.mark.parametrize("rank,heads,window,page", [(64, 6, 72, 16), (20, 2, 5, 8), (136, 9, 33, 16), (264, 3, 64, 32), (48, 1, None, 8)])
+@pytest.mark.parametrize("rank,heads,window,page", [(64, 5, 70, 16), (20, 2, 5, 8), (136, 9, 33, 16), (264, 3, 64, 32), (48, 1, None, 8)])
 def test_latent_attention_sees_exactly_its_window(rank, heads, window, page):
     """One request of 150 cached rows.  The rows just inside and just outside the window of the last tokens, the first
     rows of the sequence, a row a hundred back and the rows at the borders of pages are made to match the query twenty
@@ -285,7 +285,7 @@ def test_latent_attention_sees_exactly_its_window(rank, heads, window, page):
                 assert err < 2e-5, "mark %s, sink %s, token %d: %.3g" % (mark, sink_value, i, err)
 
 
-@pytest.mark.parametrize("rank,heads,window,page", [(64, 6, 72, 16), (48, 3, 19, 8), (128, 20, 33, 16), (256, 5, 100, 32),
+@pytest.mark.parametrize("rank,heads,window,page", [(64, 7, 75, 16), (48, 3, 19, 8), (128, 20, 33, 16), (256, 5, 100, 32),
                                                     (512, 17, None, 16), (136, 2, 40, 64)])
 def test_latent_attention_on_the_matrix_cores(rank, heads, window, page):
     """bfloat16, both copies of the latent in the pages.  Three requests in one step: a portion of 21 tokens behind 140
@@ -376,6 +376,26 @@ def test_bounded_gated_activation():
         u = torch.clamp(gu[:, inter:].double(), -1.25, 1.25)
         assert H.rel_err(got, a * torch.sigmoid(1.702 * a) * (u + 1)) < 1e-6
         assert float(gu[:, :inter].max()) > 1.25 and float(gu[:, inter:].min()) < -1.25      # the bounds were reached
+
+
+@pytest.mark.parametrize("rows,inter", [(1, 136), (8, 2048), (16, 8960), (40, 256)])
+def test_gated_product_with_the_bounded_gate_in_its_epilogue(rows, inter):
+    """The decode step's gate-up product with the bounded activation folded in, against the plain formula on the same
+    bfloat16 operands; the sizes take the kernel's ordinary tiles and the evenly dealt ones."""
+    from ginfer_amd.kernels import ops
+    g = torch.Generator().manual_seed(rows + inter)
+    x = (torch.randn((rows, 192), generator=g) * 0.5).to(torch.bfloat16)
+    w = (torch.randn((2 * inter, 192), generator=g) * 0.25).to(torch.bfloat16)
+    got = ops.gemm_skinny(x.cuda(), w.cuda(), gated=True, gate_bounds=(1.25, 1.702, 1.0)).float().cpu()
+    a = torch.clamp(x.double() @ w[:inter].double().T, max=1.25)
+    u = torch.clamp(x.double() @ w[inter:].double().T, -1.25, 1.25)
+    ref = a * torch.sigmoid(1.702 * a) * (u + 1)
+    assert float((x.double() @ w[:inter].double().T).max()) > 1.25                 # the bound was reached
+    assert H.rel_err(got, ref) < 1e-2
+    # and without bounds the same entry computes the plain SiLU gate
+    plain = ops.gemm_skinny(x.cuda(), w.cuda(), gated=True).float().cpu()
+    gate, up = x.double() @ w[:inter].double().T, x.double() @ w[inter:].double().T
+    assert H.rel_err(plain, torch.nn.functional.silu(gate) * up) < 1e-2
 
 
 # ----------------------------------------------------------------------------------------------- whole models

@@ -72,6 +72,15 @@ def test_tensor_names_shapes_and_caches():
     assert model.capturable()
 
 
+def test_a_layer_without_a_mask_sees_every_earlier_position():
+    c = copy.deepcopy(CFG)
+    del c["layers"][1]["mixer"]["mask"]
+    spec = config_from_dict(c).model_spec()
+    assert spec.layers[1].parts["mixer"].params["window"] is None
+    model = build_model(spec, torch.float32, None)
+    assert model.cache_specs()[1][1] == PagedSpec((("c", 10),), None)
+
+
 def test_one_tap_keeps_no_convolution_state():
     c = copy.deepcopy(CFG)
     c["canon"]["taps"] = 1
