@@ -436,6 +436,40 @@ def test_unequal_requests_together_with_pages_and_slots_used_again(folders, name
     assert not runner.cache.requests
 
 
+def drawn_config(seed):
+    """A configuration drawn at random: any order of the two kinds of layers, widths and ranks that are multiples of 8 or
+    not, one to nine heads, windows from one key to longer than the sequences, with and without a feed-forward."""
+    rng = np.random.RandomState(seed)
+    pick = lambda *xs: xs[rng.randint(len(xs))]
+    width = int(pick(24, 40, 52, 64, 96, 136, 200))
+    layers = []
+    for _ in range(rng.randint(1, 5)):
+        mlp = None if rng.rand() < 0.3 else FF(int(pick(16, 36, 64, 100, 192)), float(pick(0.5, 1.0, 1.5, 3.0)))
+        if rng.rand() < 0.5:
+            layers.append(("hgrn2", HG(int(rng.randint(1, 6)), int(pick(4, 8, 13, 16, 32, 48, 72)), int(pick(4, 9, 16, 24, 40, 64))), mlp))
+        else:
+            layers.append(("latent_attention", LA(int(rng.randint(1, 10)), int(pick(4, 8, 12, 16, 32, 56)), int(pick(4, 8, 20, 32, 48)),
+                                                  int(pick(8, 12, 24, 40, 80)), int(pick(8, 12, 16, 24, 40, 64, 72, 128, 160)),
+                                                  float(pick(0.1, 0.25, 0.5)), int(pick(1, 2, 7, 16, 17, 31, 64, 100))), mlp))
+    return config(width, int(pick(50, 128, 301)), int(rng.randint(1, 7)), layers, eps=float(pick(1e-6, 1e-5, 1e-4)))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("seed", range(8))
+def test_configurations_drawn_at_random(tmp_path, seed, dtype):
+    cfg = drawn_config(seed)
+    folder = make_folder(tmp_path / "m", cfg, seed=seed, edit=sharpen)
+    reqs = {"q%d" % i: H.random_tokens(n, cfg["vocab"], 200 + seed + i) for i, n in enumerate([1, 23, 70])}
+    from ginfer_amd import ModelRunner
+    page = [8, 16, 32][seed % 3]
+    runner = ModelRunner(folder, dtype=dtype, page_size=page, num_pages=-(-256 // page), max_requests=3)
+    for what, steps in (("whole", H.steps_whole(reqs)), ("decoded", H.steps_last_decoded(reqs, last=20)),
+                        ("mixed", H.steps_mixed(reqs, max_live=3, seed=seed))):
+        got = H.run_steps(runner, steps)
+        runner.cache.check()
+        compare(got, reqs, folder, TOL[dtype], "drawn configuration %d (%s) %s %s" % (seed, json.dumps(cfg), dtype, what))
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_long_decoding(folders, dtype):
     """A short prompt and 400 decoded tokens: many times through every window, the recurrence four hundred steps deep,
