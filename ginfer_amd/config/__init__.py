@@ -3,6 +3,7 @@ from .registry import (ConfigError, register_architecture, registered_architectu
 from .spec import PartSpec, LayerSpec, prenorm_layer, ScheduleEntry, ModelSpec
 from .qwen2 import Qwen2Config
 from .titozen import TitozenConfig
+from .potupel import PotupelConfig
 
 __all__ = ["ConfigError", "register_architecture", "registered_architectures", "config_class",
            "config_from_dict", "config_from_folder", "PartSpec", "LayerSpec", "prenorm_layer", "ScheduleEntry",

@@ -60,6 +60,9 @@ class ScheduleEntry:
     unless `cache_of` names an earlier entry of the schedule whose cache this run reads."""
     layer: int
     cache_of: Optional[int] = None
+    # numbers of the passes of a repeated group of layers that start right before this run: the model's `reentry` part
+    # is applied to the stream once for each (ModelSpec.reentry)
+    enter: tuple = ()
 
 
 @dataclass
@@ -76,11 +79,17 @@ class ModelSpec:
     # tensor-name prefixes of the parts outside the layers, as the architecture's checkpoints spell them (a part that is
     # not listed is spelt as its role: "embedding", "final_norm", "head")
     names: Dict[str, str] = field(default_factory=dict)
+    # what is done to the stream where a group of layers is entered again (a part of the `reentry` family), or None;
+    # tail_enter: passes that start behind the last run (a repeated group without layers at the model's end)
+    reentry: Optional[PartSpec] = None
+    tail_enter: tuple = ()
 
     def name_of(self, role):
         return self.names.get(role, role)
 
     def validate(self):
+        if self.reentry is None and (self.tail_enter or any(e.enter for e in self.schedule)):
+            raise ValueError("the schedule names passes that start anew, but the model has no re-entry part")
         for i, e in enumerate(self.schedule):
             if not 0 <= e.layer < len(self.layers):
                 raise ValueError("schedule entry %d names layer %d of %d" % (i, e.layer, len(self.layers)))

@@ -177,3 +177,35 @@ extern "C" int ga_clamped_glu(void* out, const void* gu, int tokens, int inter, 
 #undef GO
   return GA_CHECK_LAUNCH();
 }
+
+// The square of relu: out[i] = max(x[i], 0)^2, the activation of a feed-forward without a gate.  out may be x.
+template <typename T>
+__global__ __launch_bounds__(256) void relu_square_kernel(T* __restrict__ out, const T* __restrict__ x, int64_t total) {
+  constexpr int V = 16 / sizeof(T);
+  const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * V;
+  if (i + V <= total) {
+    union { uint4 u; T e[V]; } a, o;
+    a.u = *reinterpret_cast<const uint4*>(x + i);
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+      const float v = fmaxf(Num<T>::ld(&a.e[j]), 0.f);
+      Num<T>::st(&o.e[j], v * v);
+    }
+    *reinterpret_cast<uint4*>(out + i) = o.u;
+  } else {
+    for (int64_t k = i; k < total; ++k) {
+      const float v = fmaxf(Num<T>::ld(x + k), 0.f);
+      Num<T>::st(out + k, v * v);
+    }
+  }
+}
+
+extern "C" int ga_relu_square(void* out, const void* x, int64_t total, int is_bf16, hipStream_t stream) {
+  if (total <= 0) return 0;
+  if (((uintptr_t)out | (uintptr_t)x) % 16) return -1;
+  const int v = is_bf16 ? 8 : 4;
+  dim3 grid((unsigned)((total + 256 * v - 1) / (256 * v))), block(256);
+  if (is_bf16) hipLaunchKernelGGL(relu_square_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)out, (const bf16_t*)x, total);
+  else hipLaunchKernelGGL(relu_square_kernel<float>, grid, block, 0, stream, (float*)out, (const float*)x, total);
+  return GA_CHECK_LAUNCH();
+}

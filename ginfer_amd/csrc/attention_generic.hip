@@ -76,7 +76,7 @@ __global__ __launch_bounds__(64 * GA_MAX_WAVES) void paged_attention_generic_ker
     const T* __restrict__ k_pages, const T* __restrict__ v_pages,
     const int32_t* __restrict__ block_table, int table_width,
     const int32_t* __restrict__ token_entry, const int32_t* __restrict__ positions, int tokens, int nh, int nkv,
-    int hd, int page_size, int window, float scale, int tq, int hpw, int min_run) {
+    int hd, int page_size, int window, float scale, int tq, int hpw, int min_run, const float* __restrict__ sinks) {
   extern __shared__ float lds[];
   const int group = nh / nkv, head_blocks = (group + hpw - 1) / hpw;     // hpw heads of a kv group to a workgroup
   const int waves = tq * hpw, threads = blockDim.x;        // wavefronts that compute; all threads load (see the launcher)
@@ -290,7 +290,7 @@ __global__ __launch_bounds__(64 * GA_MAX_WAVES) void paged_attention_generic_ker
   }
   if (!done) return;
   T* op = out + t * out_stride + (int64_t)h * hd;
-  const float inv = 1.0f / l;
+  const float inv = 1.0f / (sinks ? l + expf(sinks[h] - m) : l);     // a sink: a score with no value, in every sum
 #pragma unroll
   for (int i = 0; i < MAX_HD / WAVE; ++i) {
     const int d = lane + i * WAVE;
@@ -443,7 +443,7 @@ __global__ __launch_bounds__(64 * (MA_MAX_COMPUTE + MA_LOADERS)) void paged_atte
     const T* __restrict__ k_pages, const T* __restrict__ v_pages,
     const int32_t* __restrict__ block_table, int table_width,
     const int32_t* __restrict__ token_entry, const int32_t* __restrict__ positions, int tokens, int nh, int nkv,
-    int page_size, int window, float scale, int tq, int hpw) {
+    int page_size, int window, float scale, int tq, int hpw, const float* __restrict__ sinks) {
   extern __shared__ float lds[];
   constexpr int hd = HD;
   constexpr int KS = HD + KPAD;                  // the layout of a tile in LDS: TileLoader
@@ -643,7 +643,7 @@ __global__ __launch_bounds__(64 * (MA_MAX_COMPUTE + MA_LOADERS)) void paged_atte
   }
   if (!done) return;
   T* op = out + t * out_stride + (int64_t)h * hd;
-  const float inv = 1.0f / l;
+  const float inv = 1.0f / (sinks ? l + expf(sinks[h] - m) : l);     // a sink: a score with no value, in every sum
 #pragma unroll
   for (int i = 0; i < NBLK; ++i)
 #pragma unroll
@@ -667,7 +667,7 @@ __global__ __launch_bounds__(64 * (HA_COMPUTE + HA_LOADERS)) void paged_attentio
     const T* __restrict__ k_pages, const T* __restrict__ v_pages,
     const int32_t* __restrict__ block_table, int table_width,
     const int32_t* __restrict__ token_entry, const int32_t* __restrict__ positions, int tokens, int nh, int nkv,
-    int page_size, int window, float scale, int min_run) {
+    int page_size, int window, float scale, int min_run, const float* __restrict__ sinks) {
   extern __shared__ float lds[];
   constexpr int KS = HD + KPAD;                  // the layout of a tile in LDS: TileLoader
   constexpr int NBLK = HD / 16;                  // blocks of 16 dimensions of the output
@@ -779,7 +779,7 @@ __global__ __launch_bounds__(64 * (HA_COMPUTE + HA_LOADERS)) void paged_attentio
   }
   if (!live) return;
   T* op = out + t * out_stride + (int64_t)h * HD;
-  const float inv = 1.0f / l;
+  const float inv = 1.0f / (sinks ? l + expf(sinks[h] - m) : l);     // a sink: a score with no value, in every sum
 #pragma unroll
   for (int i = 0; i < BPW; ++i) {
     const int blk = wave + HA_COMPUTE * i;
@@ -806,7 +806,8 @@ extern "C" int ga_paged_attention_generic(void* out, int64_t out_stride, const v
                                           const void* positions, int tokens, int nh, int nkv, int hd,
                                           int page_size, int window, float scale, int is_bf16,
                                           int tokens_per_workgroup, int few_tokens_workgroups,
-                                          int fill_workgroups, hipStream_t stream) {
+                                          int fill_workgroups, const void* sink_scores, hipStream_t stream) {
+  const float* sinks = (const float*)sink_scores;      // one score per head that every query sees beside its keys, or null
   if (tokens <= 0) return 0;
   if (hd > MAX_HD || hd <= 0 || nkv <= 0 || nh % nkv != 0 || page_size <= 0) return -1;
   const int group = nh / nkv;
@@ -860,7 +861,7 @@ extern "C" int ga_paged_attention_generic(void* out, int64_t out_stride, const v
     hipLaunchKernelGGL((paged_attention_matrix_kernel<TT, VV, HH>), grid, block, lds, stream, (TT*)out, out_stride,  \
                        (const TT*)q, q_stride, (const TT*)k_pages, (const TT*)v_pages, (const int32_t*)block_table,  \
                        table_width, (const int32_t*)token_entry, (const int32_t*)positions, tokens, nh, nkv,          \
-                       page_size, window, scale, tq, hpw);                                                           \
+                       page_size, window, scale, tq, hpw, sinks);                                                         \
   } while (0)
 #define LAUNCH_MATRIX_HD(TT, VV)                                                                                     \
   do {                                                                                                               \
@@ -912,7 +913,7 @@ extern "C" int ga_paged_attention_generic(void* out, int64_t out_stride, const v
     hipLaunchKernelGGL((paged_attention_heads_kernel<TT, VV, HH>), grid, block, lds, stream, (TT*)out, out_stride,   \
                        (const TT*)q, q_stride, (const TT*)k_pages, (const TT*)v_pages, (const int32_t*)block_table,  \
                        table_width, (const int32_t*)token_entry, (const int32_t*)positions, tokens, nh, nkv,          \
-                       page_size, window, scale, min_run);                                                           \
+                       page_size, window, scale, min_run, sinks);                                                         \
   } while (0)
 #define LAUNCH_HEADS_HD(TT, VV)                                                                                      \
   do {                                                                                                               \
@@ -964,7 +965,7 @@ extern "C" int ga_paged_attention_generic(void* out, int64_t out_stride, const v
     hipLaunchKernelGGL((paged_attention_generic_kernel<TT, VV, PP>), grid, block, lds, stream, (TT*)out, out_stride, \
                        (const TT*)q, q_stride, (const TT*)k_pages, (const TT*)v_pages, (const int32_t*)block_table,  \
                        table_width, (const int32_t*)token_entry, (const int32_t*)positions, tokens, nh, nkv, hd,      \
-                       page_size, window, scale, tq, hpw, min_run);                                                  \
+                       page_size, window, scale, tq, hpw, min_run, sinks);                                                \
   } while (0)
   if (is_bf16) {
     if (wide && pipelined) LAUNCH(bf16_t, 8, true);

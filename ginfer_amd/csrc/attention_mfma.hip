@@ -68,6 +68,12 @@ typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
 // the bare v_exp_f32: arguments here are differences to a running maximum (<= 0, or -inf), for which the
 // library routine's extra steps for denormal results buy nothing
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+// A sink: a score that every query of a head sees beside its keys' and that has no value.  sinks: one score per head
+// (natural units; the maxima here are in units of log 2) or null.  The denominator l, relative to the maximum m, with
+// the sink's share added.
+__device__ __forceinline__ float sink_sum(float l, float m, const float* __restrict__ sinks, int head) {
+  return sinks ? l + fast_exp2(sinks[head] * LOG2E - m) : l;
+}
 
 __device__ __forceinline__ bf16x8 zero8() {
   uint4 z = {0u, 0u, 0u, 0u};
@@ -401,7 +407,7 @@ __global__ __launch_bounds__(64 * DEC_WAVES) void attn_decode_split_kernel(
     const bf16_t* __restrict__ q, int64_t q_stride, const bf16_t* __restrict__ k_pages,
     const bf16_t* __restrict__ v_pages, const int32_t* __restrict__ block_table, int table_width,
     const int4* __restrict__ decode_info, int nh, int nkv, int head_blocks, int ps_shift, int window,
-    float scale, int split_keys, int num_splits) {
+    float scale, int split_keys, int num_splits, const float* __restrict__ sinks) {
   __shared__ float o_s[DEC_WAVES][HD][17];
   __shared__ float m_s[DEC_WAVES][16], l_s[DEC_WAVES][16], mx_s[16], lsum_s[16];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15, g = lane >> 4;
@@ -469,7 +475,8 @@ __global__ __launch_bounds__(64 * DEC_WAVES) void attn_decode_split_kernel(
 #pragma unroll
     for (int w = 0; w < DEC_WAVES; ++w) acc += o_s[w][d][cc];
     if (num_splits == 1) {
-      out[(int64_t)t * out_stride + (int64_t)(kvh * group + hb * 16 + cc) * HD + d] = f32_to_bf16(acc * (1.f / lsum_s[cc]));
+      const int hh = kvh * group + hb * 16 + cc;
+      out[(int64_t)t * out_stride + (int64_t)hh * HD + d] = f32_to_bf16(acc / sink_sum(lsum_s[cc], mx_s[cc], sinks, hh));
     } else {
       const int64_t slot = slot_base + (int64_t)cc * num_splits;
       part_o[slot * HD + d] = acc;
@@ -489,7 +496,8 @@ __global__ __launch_bounds__(64 * DEC_WAVES) void attn_decode_split_kernel(
 template <int EARLY>
 __global__ __launch_bounds__(64) void attn_decode_combine_kernel(
     bf16_t* __restrict__ out, int64_t out_stride, const float* __restrict__ part_o,
-    const float* __restrict__ part_ml, const int4* __restrict__ decode_info, int nh, int num_splits) {
+    const float* __restrict__ part_ml, const int4* __restrict__ decode_info, int nh, int num_splits,
+    const float* __restrict__ sinks) {
   __shared__ float w_s[MAX_SPLITS];
   const int ti = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
   const int64_t base = ((int64_t)ti * nh + head) * num_splits;
@@ -516,7 +524,7 @@ __global__ __launch_bounds__(64) void attn_decode_combine_kernel(
   }
   total = wave_sum(total);
   __syncthreads();
-  const float inv = 1.f / total;
+  const float inv = 1.f / sink_sum(total, mx, sinks, head);
   bf16_t* op = out + (int64_t)row * out_stride + (int64_t)head * HD;
   if (EARLY > 0) {
 #pragma unroll
@@ -569,7 +577,7 @@ template <int NB>
 __device__ __forceinline__ void write_rows(const f32x4 (&o)[NB][DB], const float (&m)[NB], const float (&l)[NB],
                                            bf16_t* __restrict__ out, int64_t out_stride, float* __restrict__ part_o,
                                            float* __restrict__ part_ml, const KeyPart& kp, int row0, int rows, int head,
-                                           int nh, int c, int g) {
+                                           int nh, int c, int g, const float* __restrict__ sinks) {
 #pragma unroll
   for (int nb = 0; nb < NB; ++nb) {
     const int j = nb * 16 + c;
@@ -585,7 +593,7 @@ __device__ __forceinline__ void write_rows(const f32x4 (&o)[NB][DB], const float
       }
       continue;
     }
-    const float inv = 1.f / l[nb];
+    const float inv = 1.f / sink_sum(l[nb], m[nb], sinks, head);
     bf16_t* op = out + (int64_t)(row0 + j) * out_stride + (int64_t)head * HD + g * 4;
 #pragma unroll
     for (int db = 0; db < DB; ++db) {
@@ -608,7 +616,8 @@ __global__ __launch_bounds__(64 * PREFILL_WAVES) void attn_prefill_kernel(
     const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
     const int32_t* __restrict__ block_table, int table_width, const int32_t* __restrict__ tiles, int nh,
     int nkv, int head_blocks, int hpw, int splits, int ps_shift, int window, float scale,
-    const int32_t* __restrict__ parts, float* __restrict__ part_o, float* __restrict__ part_ml) {
+    const int32_t* __restrict__ parts, float* __restrict__ part_o, float* __restrict__ part_ml,
+    const float* __restrict__ sinks) {
   extern __shared__ float lds[];          // [hpw][splits-1][NB] x { o[HD][17], m[16], l[16] }
   constexpr int STATE = HD * 17 + 32;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15, g = lane >> 4;
@@ -699,7 +708,7 @@ __global__ __launch_bounds__(64 * PREFILL_WAVES) void attn_prefill_kernel(
   } else if (!head_ok) {
     return;
   }
-  write_rows<NB>(o, m, l, out, out_stride, part_o, part_ml, kp, row0, rows, head, nh, c, g);
+  write_rows<NB>(o, m, l, out, out_stride, part_o, part_ml, kp, row0, rows, head, nh, c, g, sinks);
 }
 
 // ----------------------------------------------------------------------------- prefill, operands through LDS
@@ -775,7 +784,8 @@ __global__ __launch_bounds__(64 * PREFILL_WAVES) void attn_prefill_shared_kernel
     const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
     const int32_t* __restrict__ block_table, int table_width, const int32_t* __restrict__ tiles, int nh,
     int nkv, int head_blocks, int hpw, int splits, int ps_shift, int window, float scale,
-    const int32_t* __restrict__ parts, float* __restrict__ part_o, float* __restrict__ part_ml) {
+    const int32_t* __restrict__ parts, float* __restrict__ part_o, float* __restrict__ part_ml,
+    const float* __restrict__ sinks) {
   static_assert(STAGES == 2 || STAGES == 3, "two or three stages");
   extern __shared__ __attribute__((aligned(16))) unsigned char ring[];
   float* lds = reinterpret_cast<float*>(ring);      // after the loop: [hpw][splits-1][NB] x { o[HD][17], m[16], l[16] }
@@ -929,7 +939,7 @@ __global__ __launch_bounds__(64 * PREFILL_WAVES) void attn_prefill_shared_kernel
   } else if (!head_ok) {
     return;
   }
-  write_rows<NB>(o, m, l, out, out_stride, part_o, part_ml, kp, row0, rows, head, nh, c, g);
+  write_rows<NB>(o, m, l, out, out_stride, part_o, part_ml, kp, row0, rows, head, nh, c, g, sinks);
 }
 #endif
 
@@ -944,7 +954,7 @@ extern "C" int ga_attn_decode(void* out, int64_t out_stride, const void* q, int6
                               const void* v_pages, const void* block_table, int table_width,
                               const void* decode_info, int n_tokens, int nh, int nkv, int page_size, int window, float scale,
                               int split_keys, int num_splits, void* workspace_o, void* workspace_ml,
-                              hipStream_t stream) {
+                              const void* sinks, hipStream_t stream) {
   if (n_tokens <= 0) return 0;
   if (nkv <= 0 || nh % nkv) return -1;
   int ps_shift = 0;
@@ -959,13 +969,13 @@ extern "C" int ga_attn_decode(void* out, int64_t out_stride, const void* q, int6
                      (float*)workspace_o, (float*)workspace_ml, (const bf16_t*)q, q_stride,
                      (const bf16_t*)k_pages, (const bf16_t*)v_pages, (const int32_t*)block_table, table_width,
                      (const int4*)decode_info, nh, nkv, head_blocks, ps_shift, window, scale * LOG2E, split_keys,
-                     num_splits);
+                     num_splits, (const float*)sinks);
   int rc = GA_CHECK_LAUNCH();
   if (rc || num_splits == 1) return rc;
 #define COMBINE(EARLY)                                                                                       \
   hipLaunchKernelGGL(attn_decode_combine_kernel<EARLY>, dim3(n_tokens, nh), dim3(64), 0, stream, (bf16_t*)out, \
                      out_stride, (const float*)workspace_o, (const float*)workspace_ml,                        \
-                     (const int4*)decode_info, nh, num_splits)
+                     (const int4*)decode_info, nh, num_splits, (const float*)sinks)
   if (num_splits <= 8) COMBINE(8);
   else if (num_splits <= 16) COMBINE(16);
   else if (num_splits <= 32) COMBINE(32);
@@ -978,7 +988,7 @@ static int attn_prefill_tiles(void* out, int64_t out_stride, const void* q, int6
                               const void* v_pages, const void* block_table, int table_width, const void* tiles,
                               int n_tiles, int tile_rows, int nh, int nkv, int page_size, int window, float scale,
                               int fill_workgroups, int prefer_workgroups, const void* parts, void* part_o,
-                              void* part_ml, hipStream_t stream);
+                              void* part_ml, const void* sinks, hipStream_t stream);
 
 // parts: null, or for every tile int32 x 4 = (first key, end of keys, index of the tile's first row among the rows that
 // come in parts, part + (number of parts << 16)); a tile whose keys are dealt to several workgroups stands in `tiles` once
@@ -989,17 +999,18 @@ extern "C" int ga_attn_prefill(void* out, int64_t out_stride, const void* q, int
                                int table_width, const void* tiles, int n_tiles, int tile_rows, int nh, int nkv,
                                int page_size, int window, float scale, int fill_workgroups, int prefer_workgroups,
                                const void* parts, const void* part_rows, int n_part_rows, int num_parts, void* part_o,
-                               void* part_ml, hipStream_t stream) {
+                               void* part_ml, const void* sinks, hipStream_t stream) {
   if (n_tiles <= 0) return 0;
   if (nkv <= 0 || nh % nkv) return -1;
   if (parts && (n_part_rows <= 0 || num_parts < 2 || num_parts > 8 || !part_rows || !part_o || !part_ml)) return -8;
   if (!parts) n_part_rows = 0;
   int rc = attn_prefill_tiles(out, out_stride, q, q_stride, k_pages, v_pages, block_table, table_width, tiles, n_tiles,
                               tile_rows, nh, nkv, page_size, window, scale, fill_workgroups, prefer_workgroups, parts, part_o,
-                              part_ml, stream);
+                              part_ml, sinks, stream);
   if (rc || n_part_rows == 0) return rc;
   hipLaunchKernelGGL(attn_decode_combine_kernel<8>, dim3(n_part_rows, nh), dim3(64), 0, stream, (bf16_t*)out, out_stride,
-                     (const float*)part_o, (const float*)part_ml, (const int4*)part_rows, nh, num_parts);
+                     (const float*)part_o, (const float*)part_ml, (const int4*)part_rows, nh, num_parts,
+                     (const float*)sinks);
   return GA_CHECK_LAUNCH();
 }
 
@@ -1007,7 +1018,7 @@ static int attn_prefill_tiles(void* out, int64_t out_stride, const void* q, int6
                               const void* k_pages, const void* v_pages, const void* block_table,
                               int table_width, const void* tiles, int n_tiles, int tile_rows, int nh, int nkv,
                               int page_size, int window, float scale, int fill_workgroups, int prefer_workgroups,
-                              const void* parts, void* part_o, void* part_ml, hipStream_t stream) {
+                              const void* parts, void* part_o, void* part_ml, const void* sinks, hipStream_t stream) {
   if (tile_rows != 16 && tile_rows != 16 * PREFILL_NB) return -6;
   int ps_shift = 0;
   while ((1 << ps_shift) < page_size) ++ps_shift;
@@ -1051,7 +1062,7 @@ static int attn_prefill_tiles(void* out, int64_t out_stride, const void* q, int6
                        out_stride, (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, \
                        (const int32_t*)block_table, table_width, (const int32_t*)tiles, nh, nkv, head_blocks,  \
                        heads, streams, ps_shift, window, scale * LOG2E, (const int32_t*)parts, (float*)part_o, \
-                       (float*)part_ml);                                                                       \
+                       (float*)part_ml, (const float*)sinks);                                                  \
   } while (0)
       if (nb == 1) {
         if (stages == 3) LAUNCH_SHARED(1, 3); else LAUNCH_SHARED(1, 2);
@@ -1082,7 +1093,7 @@ static int attn_prefill_tiles(void* out, int64_t out_stride, const void* q, int6
                      (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages,           \
                      (const int32_t*)block_table, table_width, (const int32_t*)tiles, nh, nkv, head_blocks, \
                      hpw, splits, ps_shift, window, scale * LOG2E, (const int32_t*)parts, (float*)part_o,   \
-                     (float*)part_ml)
+                     (float*)part_ml, (const float*)sinks)
   if (lds > 48 * 1024) {                     // more dynamic LDS than the default limit: ask for it
     const void* fn = nb == 1 ? (const void*)attn_prefill_kernel<1> : (const void*)attn_prefill_kernel<PREFILL_NB>;
     if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) return -7;

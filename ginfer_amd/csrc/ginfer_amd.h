@@ -152,22 +152,24 @@ int ga_latent_attention_heads(void* out, int64_t out_t, int64_t out_h, void* ws_
 // ---- attention_generic.hip: every token attends to its request's pages; any head size up to 256, window or 0;
 // tokens_per_workgroup neighbouring tokens share a workgroup's tiles of keys and values (0: the library chooses; -1: the
 // same, and every request of the step has at least 8 tokens in it); few_tokens_workgroups, fill_workgroups: the two
-// thresholds by which the launcher chooses among its kernels (speed only)
+// thresholds by which the launcher chooses among its kernels (speed only); sink_scores: null, or one float per head: a
+// score that every query of the head sees beside its keys' and that has no value (it only enters the denominator)
 int ga_paged_attention_generic(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* k_pages,
                                const void* v_pages, const void* block_table, int table_width, const void* token_entry,
                                const void* positions, int tokens, int nh, int nkv, int hd, int page_size, int window,
                                float scale, int is_bf16, int tokens_per_workgroup, int few_tokens_workgroups,
-                               int fill_workgroups, hipStream_t stream);
+                               int fill_workgroups, const void* sink_scores, hipStream_t stream);
 
 // ---- attention_mfma.hip (one library per head size): bfloat16 on the matrix cores
 int ga_attn_head_dim();
 int ga_attn_prefill_max_tile_rows();
+// sinks (both entry points): null, or one float per head, a score that enters every denominator of the head
 // single new tokens; workspace_o: n_tokens * nh * num_splits * head_dim floats, workspace_ml: n_tokens * nh *
 // num_splits * 2 floats
 int ga_attn_decode(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* k_pages,
                    const void* v_pages, const void* block_table, int table_width, const void* decode_info, int n_tokens,
                    int nh, int nkv, int page_size, int window, float scale, int split_keys, int num_splits,
-                   void* workspace_o, void* workspace_ml, hipStream_t stream);
+                   void* workspace_o, void* workspace_ml, const void* sinks, hipStream_t stream);
 // rows of prompt portions, in tiles of int32 x 4 = (entry, first row of the step, rows, first position).  parts (or
 // null): per tile int32 x 4 = (first key, end of keys, index of the tile's first row among the rows that come in parts,
 // part + (number of parts << 16)): the keys of such a tile are dealt to several workgroups, whose partial results
@@ -177,7 +179,26 @@ int ga_attn_prefill(void* out, int64_t out_stride, const void* q, int64_t q_stri
                     const void* v_pages, const void* block_table, int table_width, const void* tiles, int n_tiles,
                     int tile_rows, int nh, int nkv, int page_size, int window, float scale, int fill_workgroups,
                     int prefer_workgroups, const void* parts, const void* part_rows, int n_part_rows, int num_parts, void* part_o,
-                    void* part_ml, hipStream_t stream);
+                    void* part_ml, const void* sinks, hipStream_t stream);
+
+// ---- output_norm.hip: residual[t] += scale * gain * y[t] / sqrt(mean(y[t]^2) + eps) (a norm on a sublayer's output, a
+// factor per channel behind it; gain and scale float [hidden], scale may be null); with `next` also next[t] = next_gain *
+// residual[t] / sqrt(mean(residual[t]^2) + next_eps), the rows that the following sublayer reads, in the compute dtype
+int ga_output_norm_add(void* residual, const void* y, const void* gain, const void* scale, float eps,
+                       const void* next_gain, float next_eps, void* next, int tokens, int hidden, int y_bf16,
+                       int next_bf16, hipStream_t stream);
+
+// ---- routing.hip: the `top` largest of every row of scores float [tokens, experts] (lowest index among equals) as
+// ids int32 [tokens, top], their softmax weights float [tokens, top], and the same weights as rows float [tokens,
+// experts] with zeros elsewhere; and the gated activation of experts laid side by side, gate_up [tokens, 2 * width] ->
+// out [tokens, width], column c weighted by dense[t, c / ff] (columns behind experts * ff by 1)
+int ga_route_topk(void* ids, void* weights, void* dense, const void* scores, int tokens, int experts, int top,
+                  hipStream_t stream);
+int ga_weighted_silu_mul(void* out, const void* gate_up, const void* dense, int tokens, int width, int experts, int ff,
+                         int is_bf16, hipStream_t stream);
+
+// ---- activation.hip: out[i] = max(x[i], 0)^2 over `total` elements (out may be x)
+int ga_relu_square(void* out, const void* x, int64_t total, int is_bf16, hipStream_t stream);
 
 // ---- random_fill.hip: out[i] = mean + std * normal(key, i) for n elements, float or bfloat16: the counter-based
 // generator of random_normal.h, which gives the host library (host/random_fill_host.cpp) the same bits

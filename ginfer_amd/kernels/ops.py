@@ -248,8 +248,17 @@ def _check_attention_operands(q, k_pages, v_pages, block_table, token_entry, pos
     return T
 
 
+def _check_sinks(sinks, num_heads, device):
+    """sinks: None, or float32 [num_heads]: a score that every query of a head sees beside its keys' and that has no
+    value (it enters the softmax's denominator only)."""
+    if sinks is not None:
+        _need(sinks.dtype == torch.float32 and sinks.shape == (num_heads,) and sinks.is_contiguous()
+              and sinks.device == device, "sinks must be contiguous float32 [%d] on the queries' device", num_heads)
+    return sinks
+
+
 def paged_attention_generic(q, k_pages, v_pages, block_table, token_entry, positions, num_heads, num_kv_heads,
-                            head_dim, scale, window=None, out=None, tokens_per_workgroup=0):
+                            head_dim, scale, window=None, out=None, tokens_per_workgroup=0, sinks=None):
     """q: rows of the fused projection ([T, >= nh*hd]; the first nh*hd columns are the queries).
     Token t attends to the keys of request token_entry[t] at positions
     [max(0, p - window + 1), p], p = positions[t].  Returns [T, nh*hd].  tokens_per_workgroup: how many neighbouring
@@ -259,6 +268,7 @@ def paged_attention_generic(q, k_pages, v_pages, block_table, token_entry, posit
     step; no token's result depends on it."""
     T = _check_attention_operands(q, k_pages, v_pages, block_table, token_entry, positions, num_heads,
                                   num_kv_heads, head_dim)
+    _check_sinks(sinks, num_heads, q.device)
     _need(0 < head_dim <= 256,
           "head_dim %d is not supported by the general attention kernel (up to 256)",
           head_dim)
@@ -271,7 +281,7 @@ def paged_attention_generic(q, k_pages, v_pages, block_table, token_entry, posit
         _i(block_table.shape[1]), _ptr(token_entry), _ptr(positions), _i(T), _i(num_heads), _i(num_kv_heads),
         _i(head_dim), _i(k_pages.shape[2]), _i(int(window) if window else 0), _f(scale), _i(_is_bf16(q.dtype)),
         _i(int(tokens_per_workgroup)), _i(TUNING.generic_few_tokens_workgroups), _i(TUNING.generic_fill_workgroups),
-        _stream()), "paged_attention_generic")
+        _ptr(sinks), _stream()), "paged_attention_generic")
     return out
 
 
@@ -660,12 +670,13 @@ def _decode_splits(plan, window, nkv, head_blocks):
 
 
 def paged_attention_mfma(q, k_pages, v_pages, block_table, step, num_heads, num_kv_heads, head_dim, scale,
-                         window=None, out=None):
+                         window=None, out=None, sinks=None):
     """bfloat16 attention of every token of the step on the matrix cores: single new tokens through the
     split-key kernel, rows of prompt portions through the tiled kernel."""
     T = _check_attention_operands(q, k_pages, v_pages, block_table, step.token_entry, step.positions, num_heads,
                                   num_kv_heads, head_dim)
     page_size = k_pages.shape[2]
+    _check_sinks(sinks, num_heads, q.device)
     _need(attention_mfma_supported(q.dtype, head_dim, page_size),
           "the matrix-core attention kernels take bfloat16, head sizes in steps of 16 up to 256 and page sizes that "
           "are powers of two from 8; got %s, head %d, page %d",
@@ -697,7 +708,7 @@ def paged_attention_mfma(q, k_pages, v_pages, block_table, step, num_heads, num_
         _check(lib.ga_attn_decode(
             _ptr(out), _i64(out.stride(0)), _ptr(q), _i64(q.stride(0)), _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
             _i(block_table.shape[1]), _ptr(plan["decode_info"]), _i(plan["n_decode"]), _i(num_heads), _i(num_kv_heads), _i(page_size), _i(w), _f(scale), _i(split_keys),
-            _i(num_splits), _ptr(ws_o), _ptr(ws_ml), _stream()), "attn_decode")
+            _i(num_splits), _ptr(ws_o), _ptr(ws_ml), _ptr(sinks), _stream()), "attn_decode")
     if plan["n_tiles"]:
         part_o = part_ml = None
         if plan["n_part_rows"]:
@@ -709,7 +720,7 @@ def paged_attention_mfma(q, k_pages, v_pages, block_table, step, num_heads, num_
             _i(block_table.shape[1]), _ptr(plan["tiles"]), _i(plan["n_tiles"]), _i(tile_rows), _i(num_heads), _i(num_kv_heads),
             _i(page_size), _i(w), _f(scale), _i(TUNING.prefill_fill_workgroups), _i(TUNING.prefill_prefer_workgroups),
             _ptr(plan["parts"]), _ptr(plan["part_rows"]),
-            _i(plan["n_part_rows"]), _i(plan["num_parts"]), _ptr(part_o), _ptr(part_ml), _stream()), "attn_prefill")
+            _i(plan["n_part_rows"]), _i(plan["num_parts"]), _ptr(part_o), _ptr(part_ml), _ptr(sinks), _stream()), "attn_prefill")
     return out
 
 
@@ -742,13 +753,15 @@ def _prefill_workgroups(step, tile_rows, group, nkv, head_dim, window):
     return window, nkv * (group // hpw), splits
 
 
-def paged_attention(q, k_pages, v_pages, block_table, step, num_heads, num_kv_heads, head_dim, scale, window=None):
+def paged_attention(q, k_pages, v_pages, block_table, step, num_heads, num_kv_heads, head_dim, scale, window=None,
+                    sinks=None):
     """Attention of every token of the step over its request's pages.  Chooses the kernel: the general
     one in 32-bit (fixed order of every sum: bit-identical however the work is cut); in bfloat16 the
-    matrix-core kernels where they take the shape."""
+    matrix-core kernels where they take the shape.  sinks: None, or float32 [num_heads], a score per head that
+    enters every denominator of the softmax and has no value."""
     if attention_mfma_supported(q.dtype, head_dim, k_pages.shape[2]):
         return paged_attention_mfma(q, k_pages, v_pages, block_table, step, num_heads, num_kv_heads, head_dim, scale,
-                                    window)
+                                    window, sinks=sinks)
     if step.max_q_len == 1:
         grouping = 1
     elif "static_plan" not in (step.extra or {}) and min(step.host_q_len) >= 8:
@@ -756,7 +769,7 @@ def paged_attention(q, k_pages, v_pages, block_table, step, num_heads, num_kv_he
     else:
         grouping = 0
     return paged_attention_generic(q, k_pages, v_pages, block_table, step.token_entry, step.positions, num_heads,
-                                   num_kv_heads, head_dim, scale, window, tokens_per_workgroup=grouping)
+                                   num_kv_heads, head_dim, scale, window, tokens_per_workgroup=grouping, sinks=sinks)
 
 
 # ---------------------------------------------------------------------------------------------------------------------
@@ -1009,3 +1022,77 @@ def latent_attention(qa, c_pages, block_table, step, sink, gate, heads, rank, pa
                                    _ptr(sink), _ptr(gate), _i(T), _i(heads), _i(rank), _i(page_size), _i(w),
                                    _f(scale), _i(_is_bf16(dtype)), _stream()), "latent_attention")
     return out
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# norm on a sublayer's output with a factor per channel, routing to experts, activations of feed-forwards without a gate
+
+def output_norm_add(residual, y, gain, scale, eps, next_gain=None, next_eps=None, dtype=None):
+    """residual float32 [T, H] += scale * gain * y / sqrt(mean(y^2) + eps), in place; y [T, H] float32 or bfloat16; gain
+    float32 [H]; scale float32 [H] or None.  With next_gain (float32 [H]) the rows next_gain * r / sqrt(mean(r^2) +
+    next_eps) of the new residual r come back in `dtype`: what the sublayer after this one reads."""
+    _dev(residual, y, gain, scale, next_gain)
+    _need(residual.dtype == torch.float32 and residual.dim() == 2 and residual.is_contiguous(),
+          "residual must be contiguous float32 [T, H]")
+    _need(y.shape == residual.shape and y.is_contiguous() and y.dtype in (torch.float32, torch.bfloat16),
+          "y must be contiguous float32 or bfloat16 %s, got %s %s", tuple(residual.shape), y.dtype, tuple(y.shape))
+    T, H = residual.shape
+    _f32(gain, (H,), "gain")
+    if scale is not None:
+        _f32(scale, (H,), "scale")
+    out = None
+    if next_gain is not None:
+        _f32(next_gain, (H,), "next_gain")
+        _need(next_eps is not None and dtype is not None, "the following norm needs its eps and the dtype of its rows")
+        out = torch.empty((T, H), dtype=dtype, device=residual.device)
+    lib = build.load("output_norm")
+    _check(lib.ga_output_norm_add(_ptr(residual), _ptr(y), _ptr(gain), _ptr(scale), _f(eps), _ptr(next_gain),
+                                  _f(next_eps if next_eps is not None else 0.0), _ptr(out), _i(T), _i(H), _i(_is_bf16(y.dtype)),
+                                  _i(_is_bf16(dtype)) if out is not None else _i(0), _stream()), "output_norm_add")
+    return out
+
+
+ROUTE_MAX_EXPERTS = 256
+
+
+def route_topk(scores, top):
+    """scores float32 [T, E] -> (ids int32 [T, top], weights float32 [T, top], dense float32 [T, E]): the `top` largest of
+    every row (the lowest index among equals), the softmax over the chosen scores alone, and the same weights as a row
+    over all experts with zeros at the others."""
+    _dev(scores)
+    _need(scores.dtype == torch.float32 and scores.dim() == 2 and scores.is_contiguous(), "scores must be contiguous float32 [T, E]")
+    T, E = scores.shape
+    _need(1 <= E <= ROUTE_MAX_EXPERTS and 1 <= top <= E, "routing takes 1 to %d experts and 1 <= top <= experts; got %d, top %d",
+          ROUTE_MAX_EXPERTS, E, top)
+    ids = torch.empty((T, top), dtype=torch.int32, device=scores.device)
+    weights = torch.empty((T, top), dtype=torch.float32, device=scores.device)
+    dense = torch.empty((T, E), dtype=torch.float32, device=scores.device)
+    lib = build.load("routing")
+    _check(lib.ga_route_topk(_ptr(ids), _ptr(weights), _ptr(dense), _ptr(scores), _i(T), _i(E), _i(top), _stream()), "route_topk")
+    return ids, weights, dense
+
+
+def weighted_silu_mul(gate_up, dense, ff):
+    """gate_up [T, 2 I] (gates of all experts side by side, then their ups) -> [T, I]: w * silu(gate) * up, the columns
+    [e * ff, (e + 1) * ff) weighted by dense[t, e], the columns behind the last expert's by 1."""
+    _dev(gate_up, dense)
+    _need(gate_up.dim() == 2 and gate_up.is_contiguous() and gate_up.shape[1] % 2 == 0, "gate_up must be contiguous [T, 2I]")
+    T, I = gate_up.shape[0], gate_up.shape[1] // 2
+    _need(dense.dtype == torch.float32 and dense.dim() == 2 and dense.shape[0] == T and dense.is_contiguous(),
+          "the experts' weights must be contiguous float32 [%d, E]", T)
+    E = dense.shape[1]
+    _need(ff >= 1 and E * ff <= I, "%d experts of %d columns do not fit %d", E, ff, I)
+    out = torch.empty((T, I), dtype=gate_up.dtype, device=gate_up.device)
+    lib = build.load("routing")
+    _check(lib.ga_weighted_silu_mul(_ptr(out), _ptr(gate_up), _ptr(dense), _i(T), _i(I), _i(E), _i(ff),
+                                    _i(_is_bf16(gate_up.dtype)), _stream()), "weighted_silu_mul")
+    return out
+
+
+def relu_square(x):
+    """max(x, 0)^2, in place; x contiguous float32 or bfloat16."""
+    _dev(x)
+    _need(x.is_contiguous() and x.data_ptr() % 16 == 0, "x must be contiguous at a 16-byte address")
+    lib = build.load("activation")
+    _check(lib.ga_relu_square(_ptr(x), _ptr(x), _i64(x.numel()), _i(_is_bf16(x.dtype)), _stream()), "relu_square")
+    return x

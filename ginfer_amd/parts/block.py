@@ -123,6 +123,50 @@ class OutputNormBlock(Arrangement):
         return None
 
 
+@register_arrangement("sandwich")
+class SandwichBlock(Arrangement):
+    """x <- x + out_norm1(mixer(norm1(x)));  x <- x + out_norm2(feed_forward(norm2(x))): a norm in front of every
+    sublayer and one on its output (which may bring a factor per channel along).  A layer may have no feed-forward (then
+    it has neither of that sublayer's norms).  The output norms are of a kind that offers `add_normed(residual, y,
+    then)`; the norm in front of the feed-forward is handed to the mixer's output norm as `then`, so that one launch
+    adds the mixer's result and makes the rows the feed-forward reads.  The 32-bit stream is updated in place; nothing
+    is left pending for the next block."""
+
+    roles = {"mixer": "mixer", "mixer_norm": "norm", "mixer_out_norm": "norm", "feed_forward": "feed_forward",
+             "feed_forward_norm": "norm", "feed_forward_out_norm": "norm"}
+    optional_roles = ("feed_forward", "feed_forward_norm", "feed_forward_out_norm")
+
+    def __init__(self, parts):
+        super().__init__(parts)
+        self.feed_forward = self._parts.get("feed_forward")
+        self.feed_forward_norm = self._parts.get("feed_forward_norm")
+        self.feed_forward_out_norm = self._parts.get("feed_forward_out_norm")
+        present = [p is not None for p in (self.feed_forward, self.feed_forward_norm, self.feed_forward_out_norm)]
+        if any(present) != all(present):
+            raise ValueError("a block names its feed-forward and that feed-forward's two norms together, or none of them")
+        for norm in (self.mixer_out_norm, self.feed_forward_out_norm):
+            if norm is not None and not hasattr(norm, "add_normed"):
+                raise ValueError("the output norms of this block add into the stream: %s has no add_normed"
+                                 % type(norm).__name__)
+        # the rows of the second norm come out of the first output norm's launch where that norm is a plain gain
+        self._fused_second = self.feed_forward_norm is not None and hasattr(self.feed_forward_norm, "weight") \
+            and hasattr(self.feed_forward_norm, "eps") and not getattr(self.feed_forward_norm, "has_bias", False)
+
+    def forward(self, residual, delta, step, cache):
+        n = self.mixer_norm.forward(residual, whole(delta, self.mixer_norm))
+        m = self.mixer.forward(n, step, cache)
+        if self.feed_forward is None:
+            self.mixer_out_norm.add_normed(residual, m)
+            return None
+        if self._fused_second:
+            n = self.mixer_out_norm.add_normed(residual, m, then=self.feed_forward_norm)
+        else:
+            self.mixer_out_norm.add_normed(residual, m)
+            n = self.feed_forward_norm.forward(residual, None)
+        self.feed_forward_out_norm.add_normed(residual, self.feed_forward.forward(n))
+        return None
+
+
 def whole(delta, norm=None):
     """A mixer or feed-forward may hand on float32 partial sums [parts, T, H] of a K-split product.  A norm
     that says `accepts_partial_sums` adds them up itself; for any other (or for none) they are added up here."""

@@ -15,15 +15,17 @@ class Embedding(Part):
 
     capturable = True
 
-    def __init__(self, vocab_size, hidden_size, dtype, device):
+    def __init__(self, vocab_size, hidden_size, dtype, device, weight_name="weight"):
+        """weight_name: the table's name inside the part ("" where the checkpoint names it as the part itself)."""
         self.vocab_size, self.hidden_size, self.dtype, self.device = int(vocab_size), int(hidden_size), dtype, device
+        self.weight_name = str(weight_name)
         self.weight = None
 
     def weight_specs(self):
-        return {"weight": WeightSpec((self.vocab_size, self.hidden_size))}
+        return {self.weight_name: WeightSpec((self.vocab_size, self.hidden_size))}
 
     def bind_weights(self, t):
-        self.weight = t["weight"]
+        self.weight = t[self.weight_name]
 
     def kernel_modules(self):
         return ["embedding"]

@@ -80,3 +80,86 @@ class ClampedGLU(Part):
         else:
             act = ops.clamped_glu(linear(x, self.w_gate_up), self.limit, self.alpha, self.shift)
         return linear(act, self.w_down)
+
+
+@register_feed_forward("squared_relu")
+class SquaredReLU(Part):
+    """down(relu(up(x))^2): no gate, no biases.  The tensors are named up and down."""
+
+    capturable = True
+
+    def __init__(self, hidden_size, intermediate_size, dtype, device):
+        self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
+        self.dtype, self.device = dtype, device
+        self.w_up = self.w_down = None
+
+    def weight_specs(self):
+        H, I = self.hidden_size, self.intermediate_size
+        return {"up": WeightSpec((I, H)), "down": WeightSpec((H, I))}
+
+    def bind_weights(self, t):
+        self.w_up, self.w_down = t["up"], t["down"]
+
+    def kernel_modules(self):
+        return ["activation", "gemm"] + (["gemm_skinny"] if self.dtype == torch.bfloat16 else [])
+
+    def forward(self, x):
+        return linear(ops.relu_square(linear(x, self.w_up)), self.w_down)
+
+
+@register_feed_forward("routed_glu")
+class RoutedGLU(Part):
+    """A mixture of gated feed-forwards.  Router scores z = Wr x + b in 32-bit; every token uses the `top_k` experts with
+    the largest scores, weighted by the softmax over those scores alone; an optional shared expert of its own width
+    runs for every token and is added.  Expert: down(silu(gate(x)) * up(x)), no biases.
+
+    The experts lie side by side: ONE product gives the gates and ups of all experts (and of the shared one), the
+    activation multiplies each expert's columns by the token's weight for it (zero where the token does not use it),
+    and ONE product with the down matrices laid side by side adds the experts' results up, in 32-bit.  Routing is a
+    pure function of the token's row, so a token's result does not depend on the batch.
+    Tensors: router, router.b, e<i>.gate / .up / .down, shared.gate / .up / .down."""
+
+    capturable = True
+
+    def __init__(self, hidden_size, num_experts, top_k, expert_size, dtype, device, shared_size=None, router_bias=True):
+        self.hidden_size, self.num_experts, self.top_k = int(hidden_size), int(num_experts), int(top_k)
+        self.expert_size = int(expert_size)
+        self.shared_size = int(shared_size) if shared_size else 0
+        self.router_bias = bool(router_bias)
+        if not 1 <= self.top_k <= self.num_experts <= ops.ROUTE_MAX_EXPERTS:
+            raise ValueError("routing takes 1 <= top_k <= experts <= %d, got top_k %d of %d experts"
+                             % (ops.ROUTE_MAX_EXPERTS, self.top_k, self.num_experts))
+        self.dtype, self.device = dtype, device
+        self.w_router = self.b_router = self.w_gate_up = self.w_down = None
+
+    def weight_specs(self):
+        H, F, S = self.hidden_size, self.expert_size, self.shared_size
+        specs = {"router": WeightSpec((self.num_experts, H), std=0.2, keep_32bit=True)}
+        if self.router_bias:
+            specs["router.b"] = WeightSpec((self.num_experts,), std=0.2, keep_32bit=True)
+        for e in range(self.num_experts):
+            specs.update({"e%d.gate" % e: WeightSpec((F, H)), "e%d.up" % e: WeightSpec((F, H)),
+                          "e%d.down" % e: WeightSpec((H, F))})
+        if S:
+            specs.update({"shared.gate": WeightSpec((S, H)), "shared.up": WeightSpec((S, H)), "shared.down": WeightSpec((H, S))})
+        return specs
+
+    def bind_weights(self, t):
+        self.w_router = t["router"].float().contiguous()
+        self.b_router = t["router.b"].float().contiguous() if self.router_bias else None
+        names = ["e%d" % e for e in range(self.num_experts)] + (["shared"] if self.shared_size else [])
+        self.w_gate_up = torch.cat([t[n + ".gate"] for n in names] + [t[n + ".up"] for n in names], dim=0).contiguous()
+        self.w_down = torch.cat([t[n + ".down"] for n in names], dim=1).contiguous()
+
+    def kernel_modules(self):
+        return ["routing", "gemm"] + (["gemm_skinny"] if self.dtype == torch.bfloat16 else [])
+
+    def route(self, x):
+        """(ids int32 [T, top_k], weights float32 [T, top_k], the weights as rows over all experts [T, E])."""
+        scores = ops.gemm_nt(x if x.dtype == torch.float32 else x.float(), self.w_router, self.b_router)
+        return ops.route_topk(scores, self.top_k)
+
+    def forward(self, x):
+        _, _, dense = self.route(x)
+        act = ops.weighted_silu_mul(linear(x, self.w_gate_up), dense, self.expert_size)
+        return linear(act, self.w_down)

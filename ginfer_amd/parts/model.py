@@ -6,6 +6,7 @@ import torch
 
 from . import registry
 from .base import KVCacheSpec, StateSpec
+from ..kernels import ops
 from .block import whole
 
 
@@ -70,6 +71,9 @@ class DecoderModel:
         self.embedding = registry.lookup("embedding", spec.embedding.kind)(**spec.embedding.params, **kw)
         self.final_norm = registry.lookup("norm", spec.final_norm.kind)(**spec.final_norm.params, **kw)
         self.head = registry.lookup("head", spec.head.kind)(**spec.head.params, **kw)
+        # what happens to the stream where a group of layers is entered again (schedule entries say before which runs)
+        self.reentry = (registry.lookup("reentry", spec.reentry.kind)(**spec.reentry.params, **kw)
+                        if spec.reentry is not None else None)
         self.blocks = []
         for i, ls in enumerate(spec.layers):
             arrangement = registry.lookup("arrangement", ls.arrangement)
@@ -88,6 +92,8 @@ class DecoderModel:
             nxt = self.blocks[self.schedule[i + 1].layer] if i + 1 < len(self.schedule) else None
             takes = getattr(nxt, "takes_folded_input", None)
             norm = takes() if takes is not None else None
+            if i + 1 < len(self.schedule) and self.schedule[i + 1].enter:
+                norm = None                  # the stream changes between the two runs
             self._fold_into.append(norm if getattr(self.blocks[e.layer], "folds_output", False) else None)
 
     def _build(self, role, part_spec):
@@ -106,9 +112,11 @@ class DecoderModel:
         name_of = self.spec.name_of
         out = [(name_of("embedding"), self.embedding), (name_of("final_norm"), self.final_norm),
                (name_of("head"), self.head)]
+        if self.reentry is not None:
+            out.append((name_of("reentry"), self.reentry))
         for ls, block in zip(self.spec.layers, self.blocks):
             for role, part in block.parts():
-                out.append((ls.prefix + "." + ls.name_of(role), part))
+                out.append((_join(ls.prefix, ls.name_of(role)), part))     # a role spelt "" names its tensors in the layer itself
         return out
 
     def weight_specs(self):
@@ -159,14 +167,32 @@ class DecoderModel:
         """Logits float32 [R, V] at `step.logit_rows`."""
         residual = self.embedding.forward(step.token_ids, step)
         delta = None
+        prepared = None
+        if self.reentry is not None:
+            prepared = self.reentry.prepare(residual)
         for i, e in enumerate(self.schedule):
             cache = step.caches[i]
+            for t in e.enter:                    # a pass of a repeated group of layers starts here
+                delta = self._settle(residual, delta)
+                residual = self.reentry.forward(residual, prepared, t)
             if self._fold_into[i] is not None:
                 delta = self.blocks[e.layer].forward(residual, delta, step, cache, into_norm=self._fold_into[i])
             else:
                 delta = self.blocks[e.layer].forward(residual, delta, step, cache)
+        for t in self.spec.tail_enter:
+            delta = self._settle(residual, delta)
+            residual = self.reentry.forward(residual, prepared, t)
         n = self.final_norm.forward(residual, whole(delta, self.final_norm), rows=step.logit_rows)
         return self.head.forward(n)
+
+    @staticmethod
+    def _settle(residual, delta):
+        """Adds what a block left pending into the stream."""
+        if delta is not None:
+            if isinstance(delta, ops.ScaledRows):
+                raise ValueError("a block that folds its output into the next block's norm cannot stand before a re-entry")
+            residual.add_(whole(delta).to(residual.dtype))
+        return None
 
 
 def _join(prefix, local):

@@ -3,7 +3,7 @@ reaches it, so no part knows which model it is in.  New kinds register themselve
 decorators below; the model builder looks kinds up here and nowhere else."""
 
 _REGISTRIES = {"mixer": {}, "feed_forward": {}, "norm": {}, "position": {}, "embedding": {}, "head": {},
-               "arrangement": {}, "convolution": {}}
+               "arrangement": {}, "convolution": {}, "reentry": {}}
 
 
 def _register(role, kind):
@@ -39,6 +39,10 @@ def register_head(kind):
 
 def register_convolution(kind):
     return _register("convolution", kind)
+
+
+def register_reentry(kind):
+    return _register("reentry", kind)
 
 
 def register_arrangement(kind):
