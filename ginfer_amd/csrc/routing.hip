@@ -27,6 +27,10 @@ __global__ __launch_bounds__(ROUTE_THREADS) void route_topk_kernel(const float* 
   for (int j = 0; j < PER; ++j) {
     const int e = lane + j * ROUTE_THREADS;
     z[j] = e < experts ? scores[t * experts + e] : -INFINITY;
+    // a score that is no number (the rows that pad a recorded step may hold anything) counts as the smallest: with
+    // it no comparison below would hold, the lanes would come to different winners, each strike out its own, and the
+    // next round would find no expert left
+    if (!(z[j] == z[j])) z[j] = -INFINITY;
     taken[j] = e >= experts;
   }
   for (int k = 0; k < top; ++k) {
@@ -47,7 +51,7 @@ __global__ __launch_bounds__(ROUTE_THREADS) void route_topk_kernel(const float* 
 #pragma unroll
     for (int j = 0; j < PER; ++j)
       if (lane + j * ROUTE_THREADS == at) taken[j] = true;
-    if (lane == 0) { chosen_s[k] = best; chosen_i[k] = at; }
+    if (lane == 0) { chosen_s[k] = best; chosen_i[k] = at < experts ? at : 0; }   // top <= experts: one is always left
   }
   __syncthreads();
   // softmax over the chosen scores; chosen_s[0] is the largest
