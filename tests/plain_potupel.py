@@ -91,9 +91,10 @@ def rotate(u, heads, dim, rot, first_position=0):
     return u.reshape(T, heads * dim)
 
 
-def sink_softmax_attention(q, k, v, heads, kv_heads, dim, vdim, scale):
+def sink_softmax_attention(q, k, v, heads, kv_heads, dim, vdim, scale, sink_scores=None):
     """q [T, heads*dim], k [T, kv_heads*dim], v [T, kv_heads*vdim] -> [T, heads*vdim]; causal, one added to the
-    denominator of the softmax."""
+    denominator of the softmax: a sink whose score is 0 (the design's; sink_scores gives every head another, for tests
+    of the mechanism) and which has no value."""
     T = q.shape[0]
     q = q.reshape(T, heads, dim)
     k = k.reshape(T, kv_heads, dim)
@@ -104,9 +105,10 @@ def sink_softmax_attention(q, k, v, heads, kv_heads, dim, vdim, scale):
     for h in range(heads):
         g = h // per
         s = ((q[:, h] @ k[:, g].T) * scale).masked_fill(~seen, -math.inf)
-        top = s.max(dim=-1, keepdim=True).values.clamp_min(0.0)        # the sink's score is 0
+        sink = 0.0 if sink_scores is None else float(sink_scores[h])
+        top = s.max(dim=-1, keepdim=True).values.clamp_min(sink)
         e = torch.exp(s - top)
-        out[:, h] = (e / (torch.exp(-top) + e.sum(dim=-1, keepdim=True))) @ v[:, g]
+        out[:, h] = (e / (torch.exp(sink - top) + e.sum(dim=-1, keepdim=True))) @ v[:, g]
     return out.reshape(T, heads * vdim)
 
 

@@ -1,0 +1,610 @@
+"""The Potupel decoder in the engine against its plain statement (plain_potupel.py), on the GPU: each mechanism alone,
+then whole models under every way of cutting and batching, in 32-bit and in bfloat16, at sizes of the tests' own."""
+import json
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import helpers as H
+import plain_potupel as pp
+
+pytestmark = pytest.mark.gpu
+
+
+def AT(heads, kv_heads, dim, vdim, scale, conv=None, rot=None):
+    m = dict(heads=heads, kv_heads=kv_heads, dim=dim, vdim=vdim, scale=scale)
+    if conv is not None:
+        m["conv"] = conv
+    if rot is not None:
+        m["rot"] = rot
+    return m
+
+
+def ROT(base, dims, scaling=None):
+    r = dict(base=base, dims=dims)
+    if scaling is not None:
+        r["scaling"] = dict(zip(("factor", "low", "high", "original"), scaling))
+    return r
+
+
+DENSE = lambda ff: dict(kind="dense", ff=ff)
+
+
+def MOE(experts, top, ff, shared=None):
+    m = dict(kind="moe", router=dict(experts=experts, top=top), expert=dict(ff=ff))
+    if shared is not None:
+        m["shared"] = dict(ff=shared)
+    return m
+
+
+def config(width, vocab, layers, loop=None, eps=1e-6):
+    c = dict(architecture="Potupel", vocab=vocab, width=width, norm=dict(eps=eps),
+             layers=[dict(type="attention", mixer=m, mlp=f) for m, f in layers])
+    if loop is not None:
+        c["loop"] = dict(zip(("start", "stop", "times"), loop))
+    return c
+
+
+# Sizes that differ from one another wherever the design allows it: values wider and narrower than keys and as wide,
+# one to several kv heads, one to five taps and none, the rotation on a part of a head, on all of it and absent, with and
+# without rescaled frequencies (all three branches of the rescaling are reached at these bases), loops that start at
+# the first layer or later, run once or several times, or are absent, experts with and without a shared one, every
+# expert chosen or a single one, layers without a feed-forward.
+WIDE_VALUES = config(96, 211, [
+    (AT(4, 2, 12, 20, 0.3, conv=3, rot=ROT(5000.0, 8, (4.0, 1.0, 3.0, 64))), DENSE(136)),
+    (AT(6, 3, 16, 24, 0.2, conv=2, rot=ROT(100.0, 16)), MOE(5, 2, 24, shared=40)),
+    (AT(2, 1, 8, 8, 0.5), None),
+    (AT(3, 1, 32, 40, 0.15, conv=5, rot=ROT(10.0, 2)), MOE(3, 3, 16)),
+], loop=(1, 3, 2), eps=2e-6)
+NARROW_VALUES = config(64, 150, [
+    (AT(8, 8, 16, 8, 0.25, conv=1, rot=ROT(30000.0, 12, (8.0, 1.0, 4.0, 128))), MOE(7, 1, 20, shared=12)),
+    (AT(5, 1, 24, 16, 0.2, conv=4), DENSE(72)),
+    (AT(2, 2, 48, 32, 0.1, rot=ROT(1000.0, 48)), MOE(4, 3, 8)),
+], eps=1e-5)
+ONE_LAYER_THRICE = config(40, 64, [(AT(1, 1, 16, 16, 0.25, conv=2, rot=ROT(50.0, 16)), MOE(9, 4, 8, shared=8))], loop=(0, 1, 3))
+WHOLE_LOOP_ONCE = config(48, 97, [
+    (AT(3, 3, 8, 24, 0.35, conv=6, rot=ROT(777.0, 4)), DENSE(40)),
+    (AT(4, 2, 20, 12, 0.2, conv=3), None),
+], loop=(0, 2, 1), eps=1e-4)
+CONFIGS = {"wide": (WIDE_VALUES, 8), "narrow": (NARROW_VALUES, 16), "thrice": (ONE_LAYER_THRICE, 16), "once": (WHOLE_LOOP_ONCE, 32)}
+
+
+def make_folder(path, cfg, seed, std_scale=5.0, edit=None):
+    """A model folder with random weights, stored in bfloat16 as this design's checkpoints are (so the 32-bit engine, the
+    bfloat16 engine and the plain statement all start from the same numbers); `edit(tensors)` may change them before
+    they are written."""
+    folder = H.make_model_folder(path, cfg, seed, "bfloat16", std_scale=std_scale)
+    if edit is not None:
+        from safetensors.torch import load_file, save_file
+        file = os.path.join(folder, "model.safetensors")
+        tensors = {k: v.clone() for k, v in load_file(file).items()}
+        edit(tensors)
+        save_file(tensors, file)
+    return folder
+
+
+def sharpen(tensors):
+    """Convolutions of moderate size, and queries large enough that one key takes most of a softmax in many rows (a key
+    that is wrongly seen or missed then moves the result) while other rows keep scores near zero, where the sink holds
+    a visible share; routers with wide margins, so that few choices are close calls."""
+    for name, t in tensors.items():
+        if name.endswith(".conv"):
+            t *= 0.25
+        if name.endswith(".mix.q"):
+            t *= 2.0
+        if name.endswith(".router") or name.endswith(".router.b"):
+            t *= 3.0
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    return {name: make_folder(tmp_path_factory.mktemp(name), cfg, seed=i, edit=sharpen)
+            for i, (name, (cfg, _)) in enumerate(CONFIGS.items())}
+
+
+def runner_for(folder, name, dtype, tokens=1024, max_requests=4, **kw):
+    from ginfer_amd import ModelRunner
+    ps = CONFIGS[name][1]
+    return ModelRunner(folder, dtype=dtype, page_size=ps, num_pages=-(-tokens // ps), max_requests=max_requests,
+                       max_model_len=2048, **kw)
+
+
+def requests_for(name, lengths, seed=20):
+    return {"q%d" % i: H.random_tokens(n, CONFIGS[name][0]["vocab"], seed + i) for i, n in enumerate(lengths)}
+
+
+_plain = {}
+
+
+def plain(folder, ids):
+    key = (folder, tuple(ids))
+    if key not in _plain:
+        _plain[key] = pp.logits(ids, pp.read_weights(folder), pp.read_config(folder)).numpy()
+    return _plain[key]
+
+
+def compare(got, requests, folder, tol, what, close_calls=0.0):
+    """Every row against the plain statement.  close_calls: the share of rows that may miss the tolerance (bfloat16:
+    where two experts' scores lie within rounding of each other the engine may choose the other one; that row, and
+    faintly the rows that attend to it, then differ by more than rounding)."""
+    over, first = 0, None
+    for (rid, p), row in sorted(got.items()):
+        ref = plain(folder, requests[rid])
+        assert np.isfinite(row).all(), "%s: request %s position %d: non-finite logits" % (what, rid, p)
+        err = float(np.abs(row.astype(np.float64) - ref[p]).max() / np.abs(ref).max())
+        if err > tol:
+            over += 1
+            first = first or "%s: first wrong place is request %s position %d of %d: error %.3g > %.3g" % (
+                what, rid, p, len(requests[rid]), err, tol)
+    assert over <= close_calls * len(got), "%s (%d of %d rows)" % (first, over, len(got))
+    for rid, ids in requests.items():
+        missing = [p for p in range(len(ids)) if (rid, p) not in got]
+        assert not missing, "%s: request %s lacks logits at %s" % (what, rid, missing[:8])
+
+
+# 32-bit differs from the 64-bit plain statement by the rounding of a few hundred terms per sum, which the tests' wide
+# weights, their peaked softmaxes and the layers that run several times pass on (measured: one row in 400 reaches 5e-5);
+# bfloat16 rounds every stored activation to 8 bits
+TOL = {"float32": 1e-4, "bfloat16": 6e-2}
+CLOSE = {"float32": 0.0, "bfloat16": 0.08}
+
+
+class _Step:
+    """The few arrays of a step that the kernels under test read."""
+
+    def __init__(self, q_len, q_start):
+        dev = torch.device("cuda")
+        cu = np.concatenate([[0], np.cumsum(q_len)]).astype(np.int32)
+        self.cu_tokens = torch.tensor(cu, device=dev)
+        self.q_start = torch.tensor(q_start, dtype=torch.int32, device=dev)
+        self.token_entry = torch.tensor(np.repeat(np.arange(len(q_len)), q_len), dtype=torch.int32, device=dev)
+        self.positions = torch.tensor(np.concatenate([np.arange(s, s + n) for s, n in zip(q_start, q_len)]), dtype=torch.int32,
+                                      device=dev)
+        self.num_entries = len(q_len)
+        self.host_q_len, self.host_q_start = list(q_len), list(q_start)
+        self.extra = {}
+
+    @property
+    def max_q_len(self):
+        return max(self.host_q_len)
+
+
+# ----------------------------------------------------------------------------------------------- mechanisms alone
+
+def test_output_norm_with_layer_scale_and_the_next_norm():
+    from ginfer_amd.kernels import ops
+    g = torch.Generator().manual_seed(0)
+    for width in (7, 96, 328, 1000, 4100):          # the last: longer than a workgroup keeps in registers
+        res = torch.randn((5, width), generator=g) * 3
+        y = torch.randn((5, width), generator=g) * 0.1
+        gain, scale, nxt = (torch.randn((width,), generator=g) for _ in range(3))
+        for dtype, tol in ((torch.float32, 2e-6), (torch.bfloat16, 1e-2)):
+            for with_scale in (True, False):
+                yy = y.to(dtype)
+                r = res.cuda().clone()
+                rows = ops.output_norm_add(r, yy.cuda(), gain.cuda(), scale.cuda() if with_scale else None, 1e-5,
+                                           nxt.cuda(), 3e-6, dtype)
+                want = res.double() + pp.centered_norm(yy.double(), gain.double() - 1.0, 1e-5) * (scale.double() if with_scale else 1.0)
+                assert H.rel_err(r.cpu(), want) < 2e-6
+                assert H.rel_err(rows.float().cpu(), pp.centered_norm(want, nxt.double() - 1.0, 3e-6)) < tol
+                r2 = res.cuda().clone()
+                assert ops.output_norm_add(r2, yy.cuda(), gain.cuda(), scale.cuda() if with_scale else None, 1e-5) is None
+                assert torch.equal(r2, r)
+
+
+def test_norm_with_a_gain_stored_around_zero():
+    from ginfer_amd.parts.norm import RMSNorm
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn((6, 72), generator=g) * 2
+    stored = (torch.randn((72,), generator=g) * 0.1).to(torch.bfloat16)
+    for dtype, tol in ((torch.float32, 2e-6), (torch.bfloat16, 1e-2)):
+        norm = RMSNorm(72, 1e-5, dtype, "cuda", gain_offset=1.0, weight_name="")
+        assert list(norm.weight_specs()) == [""]
+        norm.bind_weights({"": stored.cuda().to(dtype)})
+        got = norm.forward(x.cuda().clone(), None).float().cpu()
+        assert H.rel_err(got, pp.centered_norm(x.double(), stored.double(), 1e-5)) < tol
+
+
+def test_routing_chooses_the_largest_and_weighs_them_alone():
+    from ginfer_amd.kernels import ops
+    g = torch.Generator().manual_seed(2)
+    for experts, top in ((8, 3), (5, 5), (3, 1), (70, 6), (256, 9), (1, 1)):
+        z = torch.randn((37, experts), generator=g) * 2
+        z[3] = 0.25                                   # all equal: the lowest indices win
+        if experts > 2:
+            z[5, 1] = z[5, 2] = 9.0                   # two equal at the top
+        ids, weights, dense = (t.cpu() for t in ops.route_topk(z.cuda(), top))
+        ref = torch.sort(z.double(), dim=-1, descending=True, stable=True)
+        assert torch.equal(ids.long(), ref.indices[:, :top])
+        want = torch.softmax(ref.values[:, :top], dim=-1)
+        assert H.rel_err(weights, want) < 1e-6
+        rebuilt = torch.zeros((37, experts), dtype=torch.float64).scatter_(1, ids.long(), weights.double())
+        assert torch.equal(dense.double(), rebuilt)
+        assert abs(float(weights.sum(dim=-1).min()) - 1.0) < 1e-5
+
+
+def test_routing_of_a_row_that_holds_no_numbers_stays_inside_its_row():
+    """The rows that pad a recorded step may hold anything: they get some experts, and the rows beside them are as ever."""
+    from ginfer_amd.kernels import ops
+    g = torch.Generator().manual_seed(3)
+    z = torch.randn((9, 8), generator=g)
+    bad = z.clone()
+    bad[4] = float("nan")
+    bad[6, 2:5] = float("nan")
+    bad[7] = float("inf")
+    ids, weights, dense = (t.cpu() for t in ops.route_topk(bad.cuda(), 3))
+    ids0, weights0, dense0 = (t.cpu() for t in ops.route_topk(z.cuda(), 3))
+    keep = [0, 1, 2, 3, 5, 8]
+    assert torch.equal(ids[keep], ids0[keep]) and torch.equal(weights[keep], weights0[keep]) and torch.equal(dense[keep], dense0[keep])
+    assert int(ids.min()) >= 0 and int(ids.max()) < 8
+    assert all(len(set(row.tolist())) == 3 for row in ids)
+    assert not set(ids[6].tolist()) & {2, 3, 4}
+
+
+def test_gated_activation_of_experts_side_by_side_and_squared_relu():
+    from ginfer_amd.kernels import ops
+    g = torch.Generator().manual_seed(4)
+    for experts, ff, shared in ((5, 24, 40), (3, 7, 0), (1, 16, 3)):
+        width = experts * ff + shared
+        gu = torch.randn((11, 2 * width), generator=g) * 2
+        dense = torch.rand((11, experts), generator=g)
+        dense[:, 0] = 0.0
+        gu[2, :ff] = float("nan")                     # an expert that the token does not use may hold anything
+        for dtype, tol in ((torch.float32, 1e-6), (torch.bfloat16, 1e-2)):
+            a = gu.to(dtype)
+            got = ops.weighted_silu_mul(a.cuda(), dense.cuda(), ff).float().cpu()
+            gate, up = a[:, :width].double(), a[:, width:].double()
+            w = torch.ones((11, width), dtype=torch.float64)
+            w[:, :experts * ff] = dense.double().repeat_interleave(ff, dim=1)
+            want = torch.where(w == 0, torch.zeros_like(w), w * gate * torch.sigmoid(gate) * up)
+            assert H.rel_err(got, want) < tol
+    for n in (5, 64, 1031):
+        x = torch.randn((3, n), generator=g)
+        for dtype, tol in ((torch.float32, 1e-7), (torch.bfloat16, 1e-2)):
+            a = x.to(dtype)
+            assert H.rel_err(ops.relu_square(a.cuda().clone()).float().cpu(), torch.relu(a.double()) ** 2) < tol
+
+
+def _sink_case(seqs, nh, nkv, hd, ps, dtype, seed, scale, spike=None, sink_scores=None):
+    """seqs: (tokens of the step, tokens of the request with them).  A scrambled paged cache, the step's queries, and the
+    plain result with a sink of score `sink` per head."""
+    g = torch.Generator().manual_seed(seed)
+    blocks = [-(-kv // ps) for _, kv in seqs]
+    num_pages = sum(blocks) + 3
+    perm = torch.randperm(num_pages, generator=g).tolist()
+    bt = torch.full((len(seqs), max(blocks) + 1), -1, dtype=torch.int32)
+    kp = torch.full((num_pages, nkv, ps, hd), float("nan"))
+    vp = torch.full((num_pages, nkv, hd, ps), float("nan"))
+    qs, refs = [], []
+    for e, (ql, kv) in enumerate(seqs):
+        q = torch.randn((kv, nh * hd), generator=g)
+        k = torch.randn((kv, nkv * hd), generator=g)
+        v = torch.randn((kv, nkv * hd), generator=g)
+        if spike is not None:
+            c = spike(kv)
+            k.view(kv, nkv, hd)[c] = 0
+            k.view(kv, nkv, hd)[c, :, 0] = 30.0
+            q.view(kv, nh, hd)[kv - 1] = 0
+            q.view(kv, nh, hd)[kv - 1, :, 0] = 1.0 / scale       # score 30 at key c, about N(0, hd scale^2) elsewhere
+            v.view(kv, nkv, hd)[c] = 7.0
+        q, k, v = (t.to(dtype).double() for t in (q, k, v))
+        pages = [perm.pop() for _ in range(blocks[e])]
+        bt[e, :len(pages)] = torch.tensor(pages, dtype=torch.int32)
+        for c in range(kv):
+            kp[pages[c // ps], :, c % ps, :] = k[c].view(nkv, hd).float()
+            vp[pages[c // ps], :, :, c % ps] = v[c].view(nkv, hd).float()
+        refs.append(pp.sink_softmax_attention(q, k, v, nh, nkv, hd, hd, scale, sink_scores)[kv - ql:])
+        qs.append(q[kv - ql:])
+    step = _Step([q for q, _ in seqs], [kv - q for q, kv in seqs])
+    return (torch.cat(qs).to(dtype).cuda(), kp.to(dtype).cuda(), vp.to(dtype).cuda(), bt.cuda(), step), torch.cat(refs)
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.bfloat16, 2e-2)])
+@pytest.mark.parametrize("nh,nkv,hd", [(8, 1, 64), (6, 3, 16), (4, 4, 48), (3, 1, 128), (5, 5, 40)])
+@pytest.mark.parametrize("seqs", [[(1, 1), (1, 2), (2, 2), (1, 17), (33, 40)], [(1, 300), (20, 300), (1, 64), (1, 65)],
+                                  [(125, 260), (63, 63)], [(1, 1500)], [(300, 700)]])
+def test_attention_with_a_sink_in_every_kernel(dtype, tol, nh, nkv, hd, seqs):
+    """Single tokens and portions, one to hundreds of keys: with low scores the sink holds most of the weight of the
+    first rows, so a kernel that leaves it out is far off there."""
+    from ginfer_amd.kernels import ops
+    if hd % 16 and dtype == torch.bfloat16:
+        pytest.skip("the part pads heads to multiples of 16")
+    sinks = torch.zeros((nh,), dtype=torch.float32, device="cuda")
+    (q, kp, vp, bt, step), ref = _sink_case(seqs, nh, nkv, hd, 16, dtype, seed=hd + len(seqs), scale=0.05)
+    out = ops.paged_attention(q, kp, vp, bt, step, nh, nkv, hd, 0.05, None, sinks=sinks).float().cpu()
+    assert H.rel_err(out, ref) < tol
+    plain_softmax = ops.paged_attention(q, kp, vp, bt, _Step(step.host_q_len, step.host_q_start), nh, nkv, hd, 0.05, None).float().cpu()
+    if min(kv for _, kv in seqs) <= 2:
+        assert H.rel_err(plain_softmax, ref) > 0.2        # beside one or two keys the sink is no small thing
+    # other scores of the sink: one per head
+    scores = torch.linspace(-2.0, 3.0, nh)
+    (q, kp, vp, bt, step), ref = _sink_case(seqs, nh, nkv, hd, 16, dtype, seed=hd + len(seqs), scale=0.05, sink_scores=scores.tolist())
+    out = ops.paged_attention(q, kp, vp, bt, step, nh, nkv, hd, 0.05, None, sinks=scores.cuda()).float().cpu()
+    assert H.rel_err(out, ref) < tol
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("where", ["first", "page_edge", "before_page_edge", "tile_edge", "before_tile_edge", "last"])
+def test_attention_with_a_sink_finds_one_far_key(dtype, where):
+    from ginfer_amd.kernels import ops
+    nh, nkv, hd, kv = 8, 2, 32, 300
+    place = {"first": 0, "page_edge": 16 * 9, "before_page_edge": 16 * 9 - 1, "tile_edge": 64 * 3, "before_tile_edge": 95,
+             "last": kv - 1}[where]
+    sinks = torch.zeros((nh,), dtype=torch.float32, device="cuda")
+    (q, kp, vp, bt, step), ref = _sink_case([(1, kv), (20, kv)], nh, nkv, hd, 16, dtype, seed=5, scale=0.2, spike=lambda n: place)
+    out = ops.paged_attention(q, kp, vp, bt, step, nh, nkv, hd, 0.2, None, sinks=sinks).float().cpu()
+    assert H.rel_err(out, ref) < (1e-5 if dtype == torch.float32 else 2e-2)
+    assert (out[[0, 20]] - 7.0).abs().max() < 0.1
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_mixer_alone_whole_against_cut(dtype):
+    """The attention part by itself, driven with hand-made caches: a whole sequence in one step against the plain
+    mechanism, then the same sequence cut at places inside the convolution's reach, through a slot that held another
+    request before."""
+    from ginfer_amd.parts.conv_attention import ConvAttention
+    from ginfer_amd.parts.rope import RotaryNeoX
+    from ginfer_amd.parts.model import KVView, StateView
+    dt = torch.float32 if dtype == "float32" else torch.bfloat16
+    g = torch.Generator().manual_seed(7)
+    W, nh, nkv, hd, vd, taps, ps, T = 40, 4, 2, 12, 20, 4, 8, 45
+    rot = dict(base=300.0, dims=8, scaling=dict(factor=4.0, low=1.0, high=3.0, original=16))
+    position = RotaryNeoX(theta=300.0, rotary_dim=8, max_positions=128, device="cuda", scaling=rot["scaling"])
+    part = ConvAttention(W, nh, nkv, hd, vd, 0.3, dt, "cuda", taps=taps, position=position, sink=0.0)
+    names = {"q": nh * hd, "k": nkv * hd, "v": nkv * vd}
+    w = {n: (torch.randn((r, W), generator=g) * 0.3).to(torch.bfloat16) for n, r in names.items()}
+    w.update({n + ".conv": (torch.randn((r, taps), generator=g) * 0.5).to(torch.bfloat16) for n, r in names.items()})
+    w["o"] = (torch.randn((W, nh * vd), generator=g) * 0.2).to(torch.bfloat16)
+    part.bind_weights({n: t.cuda().to(torch.float32 if n.endswith(".conv") else dt) for n, t in w.items()})
+    x = torch.randn((T, W), generator=g).to(torch.bfloat16)
+    ref = pp.attention(x.double(), {"m." + n: t.double() for n, t in w.items()}, "m",
+                       dict(heads=nh, kv_heads=nkv, dim=hd, vdim=vd, scale=0.3, conv=taps, rot=rot))
+    state_spec, kv_spec = part.cache_spec()
+    pages = 12
+    kp = torch.zeros((pages, nkv, ps, part.padded), dtype=dt, device="cuda")
+    vp = torch.zeros((pages, nkv, part.padded, ps), dtype=dt, device="cuda")
+    state = torch.full((3,) + tuple(state_spec.shape), 1e4, dtype=torch.float32, device="cuda")     # what another request left
+    table = torch.tensor([[7, 2, 9, 0, 4, 11]], dtype=torch.int32, device="cuda")
+    for cuts in ([T], [1, 1, 1, 2, 5, 3, 1, 1, 29, 1]):
+        got, at = [], 0
+        for n in cuts:
+            step = _Step([n], [at])
+            slots = torch.tensor([table[0, p // ps] * ps + p % ps for p in range(at, at + n)], dtype=torch.int64, device="cuda")
+            kv = KVView(kp, vp, table, slots, ps, True)
+            sv = StateView(state, torch.tensor([1], dtype=torch.int64, device="cuda"), True)
+            got.append(part.forward(x[at:at + n].cuda().to(dt), step, [sv, kv]).float().cpu())
+            at += n
+        assert H.rel_err(torch.cat(got), ref) < (2e-5 if dtype == "float32" else 3e-2), cuts
+
+
+# ----------------------------------------------------------------------------------------------- whole models
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", list(CONFIGS))
+def test_whole_decoded_and_in_portions(folders, name, dtype):
+    """Every request whole; then most of it in one step and the rest token by token; then in portions of 1 to 64
+    tokens, and in pairs.  In 32-bit the four agree to the bit."""
+    reqs = requests_for(name, [1, 2, 5, 44, 131])
+    runner = runner_for(folders[name], name, dtype)
+    got = {}
+    for what, steps in (("whole", H.steps_whole(reqs)), ("decoded", H.steps_last_decoded(reqs, last=48)),
+                        ("portions", H.steps_portions(reqs)), ("pairs", H.steps_portions(reqs, sizes=(2,)))):
+        got[what] = H.run_steps(runner, steps)
+        runner.cache.check()
+        compare(got[what], reqs, folders[name], TOL[dtype], "%s %s %s" % (name, dtype, what), CLOSE[dtype])
+    if dtype == "float32":
+        for what in ("decoded", "portions", "pairs"):
+            for key, row in got["whole"].items():
+                assert np.array_equal(row, got[what][key]), "%s: %s differs from whole at %s" % (name, what, key)
+
+
+def test_every_run_of_a_looped_layer_against_the_plain_stream(folders):
+    """The residual stream after every run (a looped layer counts each time), in 32-bit."""
+    name = "wide"
+    ids = H.random_tokens(37, CONFIGS[name][0]["vocab"], 5)
+    runner = runner_for(folders[name], name, "float32", use_graphs=False)
+    seen = []
+    for block in runner.model.blocks:
+        def wrapped(residual, delta, step, cache, inner=block.forward, **kw):
+            out = inner(residual, delta, step, cache, **kw)
+            seen.append(residual.clone().cpu())
+            return out
+        block.forward = wrapped
+    from ginfer_amd import StepEntry
+    runner.step([StepEntry("a", ids, [0])])
+    want = pp.residual_streams(ids, pp.read_weights(folders[name]), pp.read_config(folders[name]))
+    assert len(seen) == want.shape[0] == 6
+    for i, s in enumerate(seen):
+        assert H.rel_err(s, want[i]) < 1e-5, "after run %d" % i
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["wide", "narrow", "thrice"])
+def test_unequal_requests_together_with_pages_and_slots_used_again(folders, name, dtype):
+    """Seven requests through three state slots and a pool that holds three of them: portions of some beside single
+    tokens of others, requests that sit a step out, and every page and slot used several times."""
+    reqs = requests_for(name, [70, 3, 120, 33, 64, 17, 90], seed=50)
+    steps = H.steps_mixed(reqs, max_live=3, seed=4)
+    ps = CONFIGS[name][1]
+    tokens = H.max_live_tokens(steps, round_to=ps)
+    runner = runner_for(folders[name], name, dtype, tokens=tokens, max_requests=3)
+    alone = H.run_steps(runner_for(folders[name], name, dtype), H.steps_whole(reqs)) if dtype == "float32" else None
+    for rounds in range(2):                      # the second time the steps' shapes are known and recorded
+        got = H.run_steps(runner, steps)
+        runner.cache.check()
+        compare(got, reqs, folders[name], TOL[dtype], "%s %s mixed, round %d" % (name, dtype, rounds), CLOSE[dtype])
+        if alone is not None:
+            for key, row in alone.items():
+                assert np.array_equal(row, got[key]), "%s: in a batch, %s differs from the request alone" % (name, key)
+    assert not runner.cache.requests
+
+
+def drawn_config(seed):
+    """A configuration drawn at random."""
+    rng = np.random.RandomState(seed)
+    pick = lambda *xs: xs[rng.randint(len(xs))]
+    width = int(pick(24, 40, 52, 64, 96, 136))
+    layers = []
+    n = int(rng.randint(1, 5))
+    for _ in range(n):
+        kind = rng.rand()
+        mlp = None if kind < 0.2 else DENSE(int(pick(16, 36, 64, 100))) if kind < 0.5 else \
+            MOE(int(pick(2, 3, 8, 11)), 1, int(pick(8, 12, 40)), shared=pick(None, 8, 24))
+        if mlp is not None and mlp["kind"] == "moe":
+            mlp["router"]["top"] = int(rng.randint(1, mlp["router"]["experts"] + 1))
+        kv = int(pick(1, 2, 3))
+        dim = int(pick(4, 8, 12, 16, 32, 56))
+        dims = int(pick(2, 4, dim))
+        rot = pick(None, ROT(float(pick(10.0, 1e3, 2.5e5)), dims, pick(None, (float(pick(2.0, 8.0)), 1.0, float(pick(2.0, 4.0)), int(pick(16, 64, 512))))))
+        layers.append((AT(kv * int(rng.randint(1, 4)), kv, dim, int(pick(4, 8, 20, 32, 48)), float(pick(0.1, 0.25, 0.5)),
+                          conv=pick(None, 1, 2, 4, 7), rot=rot), mlp))
+    start = int(rng.randint(0, n))
+    loop = pick(None, (start, int(rng.randint(start + 1, n + 1)), int(rng.randint(1, 4))))
+    return config(width, int(pick(50, 128, 301)), layers, loop=loop, eps=float(pick(1e-6, 1e-5, 1e-4)))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("seed", range(8))
+def test_configurations_drawn_at_random(tmp_path, seed, dtype):
+    cfg = drawn_config(seed)
+    folder = make_folder(tmp_path / "m", cfg, seed=seed, edit=sharpen)
+    reqs = {"q%d" % i: H.random_tokens(n, cfg["vocab"], 200 + seed + i) for i, n in enumerate([1, 23, 70])}
+    from ginfer_amd import ModelRunner
+    page = [8, 16, 32][seed % 3]
+    runner = ModelRunner(folder, dtype=dtype, page_size=page, num_pages=-(-256 // page), max_requests=3, max_model_len=512)
+    for what, steps in (("whole", H.steps_whole(reqs)), ("decoded", H.steps_last_decoded(reqs, last=20)),
+                        ("mixed", H.steps_mixed(reqs, max_live=3, seed=seed))):
+        got = H.run_steps(runner, steps)
+        runner.cache.check()
+        compare(got, reqs, folder, TOL[dtype], "drawn configuration %d (%s) %s %s" % (seed, json.dumps(cfg), dtype, what), CLOSE[dtype])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding(folders, dtype):
+    """A short prompt and 400 decoded tokens, recorded steps replayed throughout; the last tokens still find the first."""
+    reqs = requests_for("wide", [420], seed=70)
+    runner = runner_for(folders["wide"], "wide", dtype)
+    got = H.run_steps(runner, H.steps_last_decoded(reqs, last=400))
+    compare(got, reqs, folders["wide"], TOL[dtype], "long decoding " + dtype, CLOSE[dtype])
+    if runner.use_graphs:
+        assert runner.counts["replayed_decode"] > 300
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_far_key_decides_the_last_token(tmp_path, dtype):
+    """One layer whose keys are the tokens themselves: the query of the last token is made to match one far key (at a
+    page's edge, the first token, or the middle of a page), whose value alone then decides the logits; a model that
+    misses the key, or the sink's share in the rows where no key matches, gives other logits.  Whole, and decoded
+    through the cache."""
+    cfg = config(32, 40, [(AT(2, 1, 16, 16, 1.0), None)])
+    for place in (0, 63, 64, 200):
+        def edit(t, place=place):
+            for n in t:
+                if n.startswith("l0.norm") or n == "final.norm":
+                    t[n].zero_()
+            t["l0.ls1"].fill_(1.0)
+            e = t["embed"]
+            e.copy_((torch.randn(e.shape, generator=torch.Generator().manual_seed(1)) * 0.2).to(e.dtype))
+            e[7].zero_()
+            e[8].zero_()
+            e[7, 1] = 4.0                              # token 7: the far key (keys read coordinate 1)
+            e[8, 0] = 4.0                              # token 8, the last: the query that matches it (queries read coordinate 0)
+            t["l0.mix.q"].zero_()
+            t["l0.mix.k"].zero_()
+            t["l0.mix.q"][:, 0] = 1.0
+            t["l0.mix.k"][:, 1] = 1.0
+        folder = make_folder(tmp_path / ("m%d" % place), cfg, seed=3, std_scale=1.0, edit=edit)
+        ids = [int(x) % 6 for x in H.random_tokens(260, 40, place)]
+        ids[place] = 7
+        ids[-1] = 8
+        reqs = {"a": ids}
+        runner = runner_for(folder, "narrow", dtype, tokens=512)
+        for what, steps in (("whole", H.steps_whole(reqs)), ("decoded", H.steps_last_decoded(reqs, last=3))):
+            got = H.run_steps(runner, steps)
+            compare(got, reqs, folder, TOL[dtype], "far key at %d, %s, %s" % (place, what, dtype))
+        moved = list(ids)
+        moved[place] = 1
+        assert H.rel_err(plain(folder, moved)[-1], plain(folder, ids)[-1]) > 0.05      # the key matters in the plain statement
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_recorded_steps_equal_launched_ones(folders, dtype):
+    reqs = requests_for("wide", [60, 25, 41], seed=80)
+    steps = H.steps_mixed(reqs, max_live=3, seed=9)
+    outs = []
+    for graphs in (True, False):
+        runner = runner_for(folders["wide"], "wide", dtype, use_graphs=graphs)
+        for rounds in range(3):
+            got = H.run_steps(runner, steps)
+        outs.append(got)
+        if graphs:
+            assert runner.use_graphs and runner.counts["replayed_decode"] + runner.counts["replayed_padded"] > 0
+    for key, row in outs[0].items():
+        if dtype == "float32":
+            assert np.array_equal(row, outs[1][key]), key
+    if dtype == "bfloat16":
+        compare(outs[0], reqs, folders["wide"], TOL[dtype], "recorded", CLOSE[dtype])
+        compare(outs[1], reqs, folders["wide"], TOL[dtype], "launched", CLOSE[dtype])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_replay_program(folders, tmp_path, dtype):
+    reqs = requests_for("wide", [40, 9, 77], seed=90)
+    steps = H.steps_mixed(reqs, max_live=2, seed=2)
+    cfg_vocab = CONFIGS["wide"][0]["vocab"]
+    import plain_model
+    orig = plain_model.read_config
+    plain_model.read_config = lambda folder: {"vocab_size": cfg_vocab}          # the helper only asks for the vocabulary
+    try:
+        got = H.run_trace(folders["wide"], dtype, steps, tmp_path / "out", H.max_live_tokens(steps), page_size=16)
+    finally:
+        plain_model.read_config = orig
+    compare(got, reqs, folders["wide"], TOL[dtype], "trace replay " + dtype, CLOSE[dtype])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_greedy_generation_through_the_entry_point(folders, dtype):
+    """Engine.generate with its scheduler: five prompts through three slots under a budget of 48 tokens a step.  Every
+    token is the plain statement's greedy choice after the engine's own tokens so far (in bfloat16: or within rounding
+    of it)."""
+    from ginfer_amd import Engine, EngineConfig, SamplingParams
+    name = "narrow"
+    folder = folders[name]
+    prompts = list(requests_for(name, [3, 30, 11, 64, 1], seed=100).values())
+    eng = Engine(EngineConfig(model_path=folder, dtype=dtype, max_num_batched_tokens=48, max_num_seqs=3, max_seq_len=256,
+                              kvcache_block_size=8, num_kvcache_blocks=96))
+    outs = eng.generate(prompts, SamplingParams(max_tokens=24, ignore_eos=True))
+    cfg, w = pp.read_config(folder), pp.read_weights(folder)
+    far = 0
+    for p, o in zip(prompts, outs):
+        assert len(o.token_ids) == 24
+        logits = pp.logits((p + o.token_ids)[:-1], w, cfg)
+        for k, tok in enumerate(o.token_ids):
+            row = logits[len(p) - 1 + k]
+            best = int(torch.argmax(row))
+            gap = float(row[best] - row[tok]) / float(row.abs().max())
+            if dtype == "float32":
+                assert tok == best or gap <= 1e-5, "token %d after a prompt of %d: engine %d, plain %d (gap %.3g)" % (k, len(p), tok, best, gap)
+            else:
+                far += not (tok == best or gap <= 6e-2)
+    assert far <= 6                                  # bfloat16: a close call between two experts may move a token
+    eng.runner.cache.check()
+
+
+def test_command_line_generates(folders):
+    import subprocess
+    import sys
+    folder = folders["once"]
+    cmd = [sys.executable, os.path.join(H.ROOT, "bin", "ginfer"), "generate", "--model-path", folder, "--dtype", "float32",
+           "--prompt-ids", "1,2,3,4,5", "--max-tokens", "6", "--ignore-eos", "--max-num-seqs", "2", "--max-seq-len", "64",
+           "--num-kvcache-blocks", "16"]
+    out = subprocess.run(cmd, capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stderr[-2000:]
+    cfg, w = pp.read_config(folder), pp.read_weights(folder)
+    ids = [1, 2, 3, 4, 5]
+    for _ in range(6):
+        ids.append(int(torch.argmax(pp.logits(ids, w, cfg)[-1])))
+    assert json.loads(out.stdout.strip().splitlines()[0])["token_ids"] == ids[5:]
