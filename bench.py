@@ -71,7 +71,36 @@ def _titozen_size(width, ff, heads, kv_rank, q_rank, window, kv_heads, layers=6,
 TITOZEN_SIZES = {"1.5b": _titozen_size(1536, 8960, 12, 256, 768, 1024, 2), "7b": _titozen_size(3584, 18944, 28, 512, 1536, 2048, 4)}
 
 
+# Layer sizes for the Potupel design beside Qwen2 at equal width, heads, layers run and vocabulary (--potupel): four layers
+# of which the two in the middle run twice (six runs beside Qwen2's six layers); the first layer's feed-forward is the
+# dense one (two matrices of the width Qwen2's three have), the others route every token to 2 of 8 experts beside a shared
+# one, each a third as wide as Qwen2's feed-forward, so that a token passes as many weights as in Qwen2; keys and values
+# as wide as Qwen2's, half of a head rotated, four taps.
+def _potupel_size(width, ff, heads, kv_heads, layers=6, vocab=32768):
+    rot = dict(base=500000.0, dims=64, scaling=dict(factor=8.0, low=1.0, high=4.0, original=8192))
+    mixer = dict(heads=heads, kv_heads=kv_heads, dim=128, vdim=128, scale=128 ** -0.5, conv=4, rot=rot)
+    third = -(-ff // 3 // 64) * 64
+    moe = dict(kind="moe", router=dict(experts=8, top=2), expert=dict(ff=third), shared=dict(ff=third))
+    potupel = dict(architecture="Potupel", vocab=vocab, width=width, norm=dict(eps=1e-5), loop=dict(start=1, stop=3, times=2),
+                   layers=[dict(type="attention", mixer=dict(mixer), mlp=dict(kind="dense", ff=ff) if i == 0 else moe)
+                           for i in range(layers - 2)])
+    qwen2 = dict(SHAPE, num_hidden_layers=layers, hidden_size=width, num_attention_heads=heads, num_key_value_heads=kv_heads,
+                 head_dim=128, intermediate_size=ff, vocab_size=vocab, max_position_embeddings=32768)
+    return potupel, qwen2
+
+
+POTUPEL_SIZES = {"1.5b": _potupel_size(1536, 8960, 12, 2), "7b": _potupel_size(3584, 18944, 28, 4)}
+
+
 def compare_titozen(args):
+    return compare_designs(args, "titozen", "Titozen", args.titozen, TITOZEN_SIZES)
+
+
+def compare_potupel(args):
+    return compare_designs(args, "potupel", "Potupel", args.potupel, POTUPEL_SIZES)
+
+
+def compare_designs(args, key, name, chosen, sizes):
     """Prefill of --prefill-tokens tokens and decode steps at --batch and the --points (contexts ending at --context)
     through Engine.step, for each size and each of the two designs."""
     import torch
@@ -80,14 +109,14 @@ def compare_titozen(args):
     batches = sorted({int(p) for p in args.points.split(",") if p} | {args.batch})
     max_b = max(batches)
     g = torch.Generator().manual_seed(0)
-    out = {"metric": "prefill and decode tok/s of the Titozen design beside Qwen2 at equal sizes", "unit": "tok/s", "n_gpus": 1,
+    out = {"metric": "prefill and decode tok/s of the %s design beside Qwen2 at equal sizes" % name, "unit": "tok/s", "n_gpus": 1,
            "steps": args.steps, "warmup": args.warmup, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
            "data": "synthetic tokens, random weights", "prefill_tokens": T, "context": C, "sizes": {}}
-    for size in [x for x in args.titozen.split(",") if x]:
-        if size not in TITOZEN_SIZES:
-            sys.exit("bench.py: --titozen takes %s, got %r" % (", ".join(sorted(TITOZEN_SIZES)), size))
+    for size in [x for x in chosen.split(",") if x]:
+        if size not in sizes:
+            sys.exit("bench.py: --%s takes %s, got %r" % (key, ", ".join(sorted(sizes)), size))
         row = {}
-        for design, cfg in zip(("titozen", "qwen2"), TITOZEN_SIZES[size]):
+        for design, cfg in zip((key, "qwen2"), sizes[size]):
             engine = Engine(EngineConfig(
                 model_path=None, model_config=config_from_dict(cfg), random_seed=0, dtype=args.dtype,
                 max_num_batched_tokens=max(2048, T, C) + max_b, max_num_seqs=max_b, max_seq_len=max(T, C) + max_b + 24,
@@ -178,6 +207,9 @@ def main():
                     help="instead of the headline: prefill and decode throughput of the Titozen design at layer sizes that "
                          "resemble real models (comma-separated: %s), each beside the Qwen2 design at equal width, "
                          "feed-forward, layers and vocabulary; one JSON line" % ", ".join(sorted(TITOZEN_SIZES)))
+    ap.add_argument("--potupel", default=None, metavar="SIZES",
+                    help="instead of the headline: the same comparison for the Potupel design (comma-separated: %s)"
+                         % ", ".join(sorted(POTUPEL_SIZES)))
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this engine runs on ONE GPU; --gpus %d is not supported" % args.gpus)
@@ -188,6 +220,9 @@ def main():
 
     if args.titozen:
         print(json.dumps(compare_titozen(args)))
+        return
+    if args.potupel:
+        print(json.dumps(compare_potupel(args)))
         return
 
     shape_name, shape = SHAPES[args.shape]

@@ -1,0 +1,148 @@
+// Between a fused q|k|v projection and the attention kernels, for a mixer whose projections pass a short causal
+// convolution over time: one launch does, for every token of the step,
+//   c[ch]  = sum_j w[ch, j] * u[t - taps + 1 + j, ch]     (u: the projection's rows; those before the step's tokens come
+//                                                           from per-request state, zeros before the sequence's start)
+//   q, k:    the first rotary_dim coordinates of every head turned by the position's angle (pairs i, i + rotary_dim/2)
+//   q   ->   out[t, head * padded + d]                      (heads padded with zeros to the width the attention takes)
+//   k   ->   k_pages[page, kv head, place, d],   v -> v_pages[page, kv head, d, place]   (padded alike)
+// Keys are head_dim wide, values value_dim; both are stored `padded` wide.  A second launch moves the state on by the
+// step's tokens (a token of the first launch may read what the second overwrites).  The convolution, the rotation and
+// the sums are 32-bit; the projection's rows come in 32-bit too (U = float; or in the compute dtype), so that what is
+// cached is rounded once, at the end.  Every entry's numbers come from device arrays.
+#include "common.h"
+#include "ginfer_amd.h"
+
+#define CR_THREADS 256
+#define CR_MAX_TAPS 16
+
+template <typename T, typename U>
+__global__ __launch_bounds__(CR_THREADS) void conv_rope_kv_kernel(
+    T* __restrict__ q_out, const U* __restrict__ proj, const float* __restrict__ w, const float* __restrict__ state,
+    const int64_t* __restrict__ slots, const int32_t* __restrict__ token_entry, const int32_t* __restrict__ cu,
+    const int32_t* __restrict__ q_start, const int32_t* __restrict__ positions, const float* __restrict__ cos_t,
+    const float* __restrict__ sin_t, const int64_t* __restrict__ slot_mapping, T* __restrict__ k_pages, T* __restrict__ v_pages,
+    int nh, int nkv, int hd, int vd, int padded, int rotary_dim, int taps, int page_size, int write_kv) {
+  extern __shared__ float row[];                       // the token's convolved q | k | v, unpadded
+  const int64_t t = blockIdx.x;
+  const int width = (nh + nkv) * hd + nkv * vd;
+  const int e = token_entry[t];
+  const int local = (int)t - cu[e];
+  const bool fresh = q_start[e] == 0;
+  const float* st = taps > 1 ? state + slots[e] * (int64_t)(taps - 1) * width : nullptr;
+  for (int c = threadIdx.x; c < width; c += CR_THREADS) {
+    float acc;
+    if (w == nullptr) {
+      acc = Num<U>::ld(proj + t * width + c);
+    } else {
+      acc = 0.f;
+      for (int j = 0; j < taps; ++j) {
+        const int back = taps - 1 - j;
+        float v;
+        if (local - back >= 0) v = Num<U>::ld(proj + (t - back) * width + c);
+        else if (fresh) v = 0.f;
+        else v = st[(int64_t)(taps - 1 + local - back) * width + c];
+        acc += w[(int64_t)c * taps + j] * v;
+      }
+    }
+    row[c] = acc;
+  }
+  __syncthreads();
+  const int half = rotary_dim / 2;
+  const int pos = positions[t];
+  const float* cs = cos_t ? cos_t + (int64_t)pos * half : nullptr;
+  const float* sn = cos_t ? sin_t + (int64_t)pos * half : nullptr;
+  // q and k: (nh + nkv) heads of hd, written `padded` wide
+  int64_t page = 0, off = 0;
+  const int64_t slot = write_kv ? slot_mapping[t] : -1;
+  if (slot >= 0) slot_page(slot, page_size, page, off);
+  for (int i = threadIdx.x; i < (nh + nkv) * padded; i += CR_THREADS) {
+    const int h = i / padded, d = i - h * padded;
+    float v = 0.f;
+    if (d < hd) {
+      const float* head = row + h * hd;
+      v = head[d];
+      if (d < rotary_dim && cs != nullptr) {
+        const int j = d < half ? d : d - half;
+        const float a = head[j], b = head[j + half];
+        v = d < half ? a * cs[j] - b * sn[j] : b * cs[j] + a * sn[j];
+      }
+    }
+    if (h < nh) {
+      Num<T>::st(q_out + t * (int64_t)nh * padded + i, v);
+    } else if (slot >= 0) {
+      const int g = h - nh;
+      Num<T>::st(k_pages + ((page * nkv + g) * page_size + off) * padded + d, v);
+    }
+  }
+  if (slot >= 0) {
+    const float* vals = row + (nh + nkv) * hd;
+    for (int i = threadIdx.x; i < nkv * padded; i += CR_THREADS) {
+      const int g = i / padded, d = i - g * padded;
+      Num<T>::st(v_pages + ((page * nkv + g) * padded + d) * page_size + off, d < vd ? vals[g * vd + d] : 0.f);
+    }
+  }
+}
+
+// one thread per (entry, channel): new state k <- the projection's row n - (taps - 1) + k of the entry's n tokens, or, where
+// that lies before the step, old state n + k (read before it is written: it lies above k), or zero for a fresh request
+template <typename T>
+__global__ __launch_bounds__(CR_THREADS) void conv_state_update_kernel(float* __restrict__ state, const T* __restrict__ proj,
+                                                                        const int64_t* __restrict__ slots,
+                                                                        const int32_t* __restrict__ cu,
+                                                                        const int32_t* __restrict__ q_start, int width, int taps) {
+  const int e = blockIdx.x;
+  const int first = cu[e], n = cu[e + 1] - first;
+  if (n <= 0) return;
+  const bool fresh = q_start[e] == 0;
+  float* st = state + slots[e] * (int64_t)(taps - 1) * width;
+  for (int c = blockIdx.y * CR_THREADS + threadIdx.x; c < width; c += gridDim.y * CR_THREADS) {
+    for (int k = 0; k < taps - 1; ++k) {
+      const int local = n - (taps - 1) + k;
+      float v;
+      if (local >= 0) v = Num<T>::ld(proj + (int64_t)(first + local) * width + c);
+      else if (fresh) v = 0.f;
+      else v = st[(int64_t)(n + k) * width + c];
+      st[(int64_t)k * width + c] = v;
+    }
+  }
+}
+
+extern "C" int ga_conv_rope_kv(void* q_out, const void* proj, const void* w, void* state, const void* slots,
+                               const void* token_entry, const void* cu, const void* q_start, const void* positions,
+                               const void* cos_t, const void* sin_t, const void* slot_mapping, void* k_pages, void* v_pages,
+                               int tokens, int entries, int nh, int nkv, int hd, int vd, int padded, int rotary_dim, int taps,
+                               int page_size, int write_kv, int update_state, int is_bf16, int proj_bf16, hipStream_t stream) {
+  if (tokens <= 0) return 0;
+  if (nh <= 0 || nkv <= 0 || hd <= 0 || vd <= 0 || padded < hd || padded < vd || page_size <= 0) return -1;
+  if (taps < 1 || taps > CR_MAX_TAPS || (w == nullptr && taps != 1)) return -2;
+  if (taps > 1 && (state == nullptr || slots == nullptr)) return -3;
+  if (rotary_dim < 0 || rotary_dim % 2 || rotary_dim > hd || (rotary_dim > 0) != (cos_t != nullptr) || (cos_t == nullptr) != (sin_t == nullptr)) return -4;
+  if (write_kv && (!slot_mapping || !k_pages || !v_pages)) return -5;
+  const int width = (nh + nkv) * hd + nkv * vd;
+  const size_t lds = (size_t)width * sizeof(float);
+  if (lds > 64 * 1024) return -6;
+#define GO(T, U)                                                                                                       \
+  do {                                                                                                                 \
+    if (lds > 48 * 1024 && hipFuncSetAttribute((const void*)conv_rope_kv_kernel<T, U>,                                 \
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)    \
+      return -7;                                                                                                       \
+    hipLaunchKernelGGL((conv_rope_kv_kernel<T, U>), dim3(tokens), dim3(CR_THREADS), lds, stream, (T*)q_out, (const U*)proj, \
+                       (const float*)w, (const float*)state, (const int64_t*)slots, (const int32_t*)token_entry,       \
+                       (const int32_t*)cu, (const int32_t*)q_start, (const int32_t*)positions, (const float*)cos_t,    \
+                       (const float*)sin_t, (const int64_t*)slot_mapping, (T*)k_pages, (T*)v_pages, nh, nkv, hd, vd,   \
+                       padded, rotary_dim, taps, page_size, write_kv);                                                 \
+    int rc = GA_CHECK_LAUNCH();                                                                                        \
+    if (rc) return rc;                                                                                                 \
+    if (update_state && taps > 1 && entries > 0) {                                                                     \
+      int cols = (width + CR_THREADS - 1) / CR_THREADS;                                                                \
+      if (cols > 64) cols = 64;                                                                                        \
+      hipLaunchKernelGGL(conv_state_update_kernel<U>, dim3(entries, cols), dim3(CR_THREADS), 0, stream, (float*)state, \
+                         (const U*)proj, (const int64_t*)slots, (const int32_t*)cu, (const int32_t*)q_start, width,    \
+                         taps);                                                                                        \
+    }                                                                                                                  \
+  } while (0)
+  if (!is_bf16 && proj_bf16) return -8;
+  if (is_bf16 && proj_bf16) GO(bf16_t, bf16_t); else if (is_bf16) GO(bf16_t, float); else GO(float, float);
+#undef GO
+  return GA_CHECK_LAUNCH();
+}

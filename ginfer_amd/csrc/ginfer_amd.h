@@ -181,6 +181,19 @@ int ga_attn_prefill(void* out, int64_t out_stride, const void* q, int64_t q_stri
                     int prefer_workgroups, const void* parts, const void* part_rows, int n_part_rows, int num_parts, void* part_o,
                     void* part_ml, const void* sinks, hipStream_t stream);
 
+// ---- conv_rope_kv.hip: behind a fused q|k|v projection proj [tokens, (nh + nkv) hd + nkv vd] whose channels pass a
+// causal convolution of `taps` taps over time (w float [channels, taps], or null with taps 1: none; state float [slots,
+// taps - 1, channels]: a request's last projected rows): convolution, rotation of the first rotary_dim coordinates of
+// q's and k's heads (cos_t, sin_t float [positions, rotary_dim / 2], or null with rotary_dim 0), q into q_out [tokens, nh
+// * padded], k and v into their pages (k [pages, nkv, page_size, padded], v [pages, nkv, padded, page_size]), heads
+// padded with zeros; then (update_state) a second launch moves the state on by the step's tokens; proj may be float
+// beside a bfloat16 compute dtype (proj_bf16 0, is_bf16 1)
+int ga_conv_rope_kv(void* q_out, const void* proj, const void* w, void* state, const void* slots, const void* token_entry,
+                    const void* cu, const void* q_start, const void* positions, const void* cos_t, const void* sin_t,
+                    const void* slot_mapping, void* k_pages, void* v_pages, int tokens, int entries, int nh, int nkv, int hd,
+                    int vd, int padded, int rotary_dim, int taps, int page_size, int write_kv, int update_state, int is_bf16,
+                    int proj_bf16, hipStream_t stream);
+
 // ---- output_norm.hip: residual[t] += scale * gain * y[t] / sqrt(mean(y[t]^2) + eps) (a norm on a sublayer's output, a
 // factor per channel behind it; gain and scale float [hidden], scale may be null); with `next` also next[t] = next_gain *
 // residual[t] / sqrt(mean(residual[t]^2) + next_eps), the rows that the following sublayer reads, in the compute dtype

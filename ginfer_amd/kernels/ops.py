@@ -1096,3 +1096,55 @@ def relu_square(x):
     lib = build.load("activation")
     _check(lib.ga_relu_square(_ptr(x), _ptr(x), _i64(x.numel()), _i(_is_bf16(x.dtype)), _stream()), "relu_square")
     return x
+
+
+def conv_rope_kv(proj, weight, state, slots, step, cos, sin, slot_mapping, k_pages, v_pages, num_heads, num_kv_heads, head_dim,
+                 value_dim, padded, dtype, write_kv=True, update_state=True):
+    """Behind a fused q|k|v projection whose channels pass a short causal convolution: proj [T, (nh + nkv) hd + nkv vd] in
+    the compute dtype `dtype` or in float32; weight float32 [channels, taps] (None: no convolution); state float32 [slots, taps - 1, channels]
+    (None for one tap) and slots int64 [entries]; cos, sin float32 [positions, rotary_dim / 2] (None: no rotation).
+    Returns q [T, nh * padded], heads padded with zeros, and writes k and v (padded alike) into the pages at slot_mapping;
+    moves the state on by the step's tokens."""
+    _dev(proj, weight, state, slots, cos, sin, slot_mapping, k_pages, v_pages)
+    T = proj.shape[0]
+    C = (num_heads + num_kv_heads) * head_dim + num_kv_heads * value_dim
+    _need(proj.dim() == 2 and proj.shape[1] == C and proj.is_contiguous() and proj.dtype in (torch.float32, torch.bfloat16),
+          "proj must be contiguous float32 or bfloat16 [T, %d], got %s %s", C, proj.dtype, tuple(proj.shape))
+    _need(C * 4 <= 64 * 1024, "this kernel keeps a token's %d channels in 64 KB of LDS", C)
+    _need(padded >= head_dim and padded >= value_dim, "heads padded to %d do not hold %d / %d", padded, head_dim, value_dim)
+    taps = 1
+    if weight is not None:
+        _need(weight.dim() == 2 and weight.shape[0] == C and 1 <= weight.shape[1] <= SHORT_CONV_MAX_TAPS,
+              "the convolution's weight must be [%d, taps <= %d], got %s", C, SHORT_CONV_MAX_TAPS, tuple(weight.shape))
+        taps = weight.shape[1]
+        _f32(weight, (C, taps), "weight")
+    E = step.cu_tokens.shape[0] - 1
+    for name, a, n in (("token_entry", step.token_entry, T), ("cu_tokens", step.cu_tokens, E + 1), ("q_start", step.q_start, E),
+                       ("positions", step.positions, T)):
+        _need(a.dtype == torch.int32 and a.shape == (n,) and a.is_contiguous(), "%s must be contiguous int32 [%d]", name, n)
+    if taps > 1:
+        _need(state is not None and state.dtype == torch.float32 and state.dim() == 3 and state.is_contiguous()
+              and tuple(state.shape[1:]) == (taps - 1, C), "state must be contiguous float32 [slots, %d, %d]", taps - 1, C)
+        _need(slots.dtype == torch.int64 and slots.shape == (E,) and slots.is_contiguous(), "slots must be contiguous int64 [%d]", E)
+    rotary_dim = 0
+    if cos is not None:
+        _need(sin is not None and cos.dtype == torch.float32 and sin.dtype == torch.float32 and cos.shape == sin.shape
+              and cos.dim() == 2 and cos.is_contiguous() and sin.is_contiguous(), "cos and sin must be contiguous float32 [P, rotary_dim/2]")
+        rotary_dim = 2 * cos.shape[1]
+        _need(0 < rotary_dim <= head_dim, "rotary_dim %d must lie in (0, head_dim %d]", rotary_dim, head_dim)
+    page_size = 1
+    if write_kv:
+        _need(slot_mapping is not None and slot_mapping.dtype == torch.int64 and slot_mapping.shape == (T,)
+              and slot_mapping.is_contiguous(), "slot_mapping must be contiguous int64 [T]")
+        page_size = _check_pages(k_pages, v_pages, dtype, num_kv_heads, padded)
+    _need(proj.dtype in (dtype, torch.float32), "proj must be %s or float32", dtype)
+    q = torch.empty((T, num_heads * padded), dtype=dtype, device=proj.device)
+    lib = build.load("conv_rope_kv")
+    _check(lib.ga_conv_rope_kv(_ptr(q), _ptr(proj), _ptr(weight), _ptr(state), _ptr(slots), _ptr(step.token_entry),
+                               _ptr(step.cu_tokens), _ptr(step.q_start), _ptr(step.positions), _ptr(cos), _ptr(sin),
+                               _ptr(slot_mapping), _ptr(k_pages), _ptr(v_pages), _i(T), _i(E), _i(num_heads), _i(num_kv_heads),
+                               _i(head_dim), _i(value_dim), _i(padded), _i(rotary_dim), _i(taps), _i(page_size),
+                               _i(1 if write_kv else 0), _i(1 if update_state else 0), _i(_is_bf16(dtype)),
+                               _i(_is_bf16(proj.dtype)), _stream()),
+           "conv_rope_kv")
+    return q

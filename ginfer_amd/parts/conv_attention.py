@@ -20,9 +20,10 @@ class ConvAttention(Part):
     paged cache, scores times `scale`; `sink`: a score that every query sees beside its keys' and that has no value
     (None: a plain softmax); Wo on the heads' results.  Keys are head_dim wide, values value_dim.
 
-    The attention kernels take one head size, so inside the part every head is `padded` = the wider of the two widths,
-    rounded up to 16: the stacked projection matrix has rows of zeros where a head is narrower, the convolution's
-    weights and Wo's columns likewise.  What the zeros add to a score or a result is exactly nothing."""
+    The attention kernels take one head size, so behind the projection every head is `padded` = the wider of the two
+    widths, rounded up to 16: one kernel convolves, rotates and lays q out so, and writes keys and values so into their
+    pages, with zeros where a head is narrower; Wo has columns of zeros there.  What the zeros add to a score or a
+    result is exactly nothing."""
 
     capturable = True
 
@@ -49,8 +50,8 @@ class ConvAttention(Part):
         self.names = dict(q="q", k="k", v="v", o="o", conv="conv")
         self.names.update(names or {})
         self.dtype, self.device = dtype, device
-        self.width = (self.nh + 2 * self.nkv) * self.padded
-        self.w_qkv = self.w_conv = self.w_o = self.sinks = self._no_rotation = None
+        self.width = (self.nh + self.nkv) * self.hd + self.nkv * self.vd        # the projection's channels
+        self.w_qkv = self.w_conv = self.w_o = self.sinks = None
 
     def cache_spec(self):
         """[the convolution's state (or None), the pages of keys and values]."""
@@ -77,21 +78,16 @@ class ConvAttention(Part):
 
     def bind_weights(self, t):
         n = self.names
-        heads = {"q": (self.nh, self.hd), "k": (self.nkv, self.hd), "v": (self.nkv, self.vd)}
-        self.w_qkv = torch.cat([self._padded_rows(t[n[r]], *heads[r]) for r in ("q", "k", "v")], dim=0).contiguous()
+        self.w_qkv = torch.cat([t[n[r]] for r in ("q", "k", "v")], dim=0).contiguous()
         if self.has_conv:
-            self.w_conv = torch.cat([self._padded_rows(t[n[r] + "." + n["conv"]].float(), *heads[r])
-                                     for r in ("q", "k", "v")], dim=0).contiguous()
+            self.w_conv = torch.cat([t[n[r] + "." + n["conv"]].float() for r in ("q", "k", "v")], dim=0).contiguous()
         w_o = t[n["o"]]
         self.w_o = self._padded_rows(w_o.t().contiguous(), self.nh, self.vd).t().contiguous()
         dev = self.w_qkv.device
         self.sinks = None if self.sink is None else torch.full((self.nh,), self.sink, dtype=torch.float32, device=dev)
-        if self.position is None:                # the cache-writing kernel rotates by tables: angle zero everywhere
-            self._no_rotation = (torch.ones((1, 1), dtype=torch.float32, device=dev),
-                                 torch.zeros((1, 1), dtype=torch.float32, device=dev))
 
     def kernel_modules(self):
-        mods = ["rope_kv", "attention_generic", "gemm", "short_conv"]
+        mods = ["conv_rope_kv", "attention_generic", "gemm"]
         if self.dtype == torch.bfloat16:
             mods += ["gemm_skinny"]
             if self.padded in ops.MFMA_HEAD_DIMS:
@@ -100,24 +96,12 @@ class ConvAttention(Part):
 
     def forward(self, x, step, cache):
         state, kv = cache
-        if self.has_conv:
-            # the convolution works on 32-bit rows and hands on the compute dtype
-            proj = linear(x, self.w_qkv, None, out_dtype=torch.float32)
-            if state is None:
-                qkv = ops.short_conv(proj, self.w_conv, None, None, step, self.dtype, add_input=False)
-            else:
-                qkv = ops.short_conv(proj, self.w_conv, state.state, state.slots, step, self.dtype, add_input=False,
-                                     update=state.owner)
-        else:
-            qkv = linear(x, self.w_qkv, None)
-        if self.position is not None:
-            cos, sin = self.position.tables()
-            positions = step.positions
-        else:
-            cos, sin = self._no_rotation
-            positions = torch.zeros_like(step.positions)
-        ops.rope_kv_write(qkv, positions, cos, sin, kv.slot_mapping, kv.k_pages, kv.v_pages, self.nh, self.nkv,
-                          self.padded, write_kv=kv.owner)
-        a = ops.paged_attention(qkv, kv.k_pages, kv.v_pages, kv.block_table, step, self.nh, self.nkv, self.padded,
+        cos, sin = self.position.tables() if self.position is not None else (None, None)
+        # the projection's rows stay 32-bit until they are convolved and rotated: what is cached is rounded once
+        q = ops.conv_rope_kv(linear(x, self.w_qkv, None, out_dtype=torch.float32), self.w_conv, None if state is None else state.state,
+                             None if state is None else state.slots, step, cos, sin, kv.slot_mapping, kv.k_pages, kv.v_pages,
+                             self.nh, self.nkv, self.hd, self.vd, self.padded, self.dtype, write_kv=kv.owner,
+                             update_state=state is not None and state.owner)
+        a = ops.paged_attention(q, kv.k_pages, kv.v_pages, kv.block_table, step, self.nh, self.nkv, self.padded,
                                 self.scale, self.window, sinks=self.sinks)
         return linear(a, self.w_o, None)
