@@ -1,5 +1,6 @@
 // Between a fused q|k|v projection and the attention kernels, for a mixer whose projections pass a short causal
 // convolution over time: one launch does, for every token of the step,
+// (a workgroup per token and head)
 //   c[ch]  = sum_j w[ch, j] * u[t - taps + 1 + j, ch]     (u: the projection's rows; those before the step's tokens come
 //                                                           from per-request state, zeros before the sequence's start)
 //   q, k:    the first rotary_dim coordinates of every head turned by the position's angle (pairs i, i + rotary_dim/2)
@@ -13,28 +14,37 @@
 #include "ginfer_amd.h"
 
 #define CR_THREADS 256
+#define CR_HEAD_THREADS 256       // channels of a head (padded): the attention kernels take up to 256
 #define CR_MAX_TAPS 16
 
+// grid (tokens, nh + 2 nkv): a workgroup per token and head (q heads, then k heads, then v heads), a thread per channel
 template <typename T, typename U>
-__global__ __launch_bounds__(CR_THREADS) void conv_rope_kv_kernel(
+__global__ __launch_bounds__(CR_HEAD_THREADS) void conv_rope_kv_kernel(
     T* __restrict__ q_out, const U* __restrict__ proj, const float* __restrict__ w, const float* __restrict__ state,
     const int64_t* __restrict__ slots, const int32_t* __restrict__ token_entry, const int32_t* __restrict__ cu,
     const int32_t* __restrict__ q_start, const int32_t* __restrict__ positions, const float* __restrict__ cos_t,
     const float* __restrict__ sin_t, const int64_t* __restrict__ slot_mapping, T* __restrict__ k_pages, T* __restrict__ v_pages,
     int nh, int nkv, int hd, int vd, int padded, int rotary_dim, int taps, int page_size, int write_kv) {
-  extern __shared__ float row[];                       // the token's convolved q | k | v, unpadded
+  __shared__ float head[CR_HEAD_THREADS];              // the head's convolved channels
   const int64_t t = blockIdx.x;
+  const int h = blockIdx.y, d = threadIdx.x;
+  const bool is_q = h < nh, is_k = !is_q && h < nh + nkv;
+  const int g = is_q ? h : is_k ? h - nh : h - nh - nkv;                // the head among its kind
+  const int own = (is_q || is_k) ? hd : vd;                             // its channels
+  const int first = is_q ? g * hd : is_k ? (nh + g) * hd : (nh + nkv) * hd + g * vd;
   const int width = (nh + nkv) * hd + nkv * vd;
-  const int e = token_entry[t];
-  const int local = (int)t - cu[e];
-  const bool fresh = q_start[e] == 0;
-  const float* st = taps > 1 ? state + slots[e] * (int64_t)(taps - 1) * width : nullptr;
-  for (int c = threadIdx.x; c < width; c += CR_THREADS) {
-    float acc;
+  const int64_t slot = (write_kv && !is_q) ? slot_mapping[t] : -1;
+  if (!is_q && slot < 0) return;                       // nothing to write for this token
+  float acc = 0.f;
+  if (d < own) {
+    const int c = first + d;
     if (w == nullptr) {
       acc = Num<U>::ld(proj + t * width + c);
     } else {
-      acc = 0.f;
+      const int e = token_entry[t];
+      const int local = (int)t - cu[e];
+      const bool fresh = q_start[e] == 0;
+      const float* st = taps > 1 ? state + slots[e] * (int64_t)(taps - 1) * width : nullptr;
       for (int j = 0; j < taps; ++j) {
         const int back = taps - 1 - j;
         float v;
@@ -44,43 +54,27 @@ __global__ __launch_bounds__(CR_THREADS) void conv_rope_kv_kernel(
         acc += w[(int64_t)c * taps + j] * v;
       }
     }
-    row[c] = acc;
   }
-  __syncthreads();
-  const int half = rotary_dim / 2;
-  const int pos = positions[t];
-  const float* cs = cos_t ? cos_t + (int64_t)pos * half : nullptr;
-  const float* sn = cos_t ? sin_t + (int64_t)pos * half : nullptr;
-  // q and k: (nh + nkv) heads of hd, written `padded` wide
-  int64_t page = 0, off = 0;
-  const int64_t slot = write_kv ? slot_mapping[t] : -1;
-  if (slot >= 0) slot_page(slot, page_size, page, off);
-  for (int i = threadIdx.x; i < (nh + nkv) * padded; i += CR_THREADS) {
-    const int h = i / padded, d = i - h * padded;
-    float v = 0.f;
-    if (d < hd) {
-      const float* head = row + h * hd;
-      v = head[d];
-      if (d < rotary_dim && cs != nullptr) {
-        const int j = d < half ? d : d - half;
-        const float a = head[j], b = head[j + half];
-        v = d < half ? a * cs[j] - b * sn[j] : b * cs[j] + a * sn[j];
-      }
-    }
-    if (h < nh) {
-      Num<T>::st(q_out + t * (int64_t)nh * padded + i, v);
-    } else if (slot >= 0) {
-      const int g = h - nh;
-      Num<T>::st(k_pages + ((page * nkv + g) * page_size + off) * padded + d, v);
+  const bool rotate = (is_q || is_k) && cos_t != nullptr;
+  if (rotate) {
+    head[d] = acc;
+    __syncthreads();
+    if (d < rotary_dim) {
+      const int half = rotary_dim / 2, j = d < half ? d : d - half;
+      const int64_t at = (int64_t)positions[t] * half + j;
+      const float a = head[j], b = head[j + half], c = cos_t[at], s = sin_t[at];
+      acc = d < half ? a * c - b * s : b * c + a * s;
     }
   }
-  if (slot >= 0) {
-    const float* vals = row + (nh + nkv) * hd;
-    for (int i = threadIdx.x; i < nkv * padded; i += CR_THREADS) {
-      const int g = i / padded, d = i - g * padded;
-      Num<T>::st(v_pages + ((page * nkv + g) * padded + d) * page_size + off, d < vd ? vals[g * vd + d] : 0.f);
-    }
+  if (d >= padded) return;                             // (acc is zero from a head's own width on)
+  if (is_q) {
+    Num<T>::st(q_out + (t * nh + g) * (int64_t)padded + d, acc);
+    return;
   }
+  int64_t page, off;
+  slot_page(slot, page_size, page, off);
+  if (is_k) Num<T>::st(k_pages + ((page * nkv + g) * page_size + off) * padded + d, acc);
+  else Num<T>::st(v_pages + ((page * nkv + g) * padded + d) * page_size + off, acc);
 }
 
 // one thread per (entry, channel): new state k <- the projection's row n - (taps - 1) + k of the entry's n tokens, or, where
@@ -119,18 +113,18 @@ extern "C" int ga_conv_rope_kv(void* q_out, const void* proj, const void* w, voi
   if (rotary_dim < 0 || rotary_dim % 2 || rotary_dim > hd || (rotary_dim > 0) != (cos_t != nullptr) || (cos_t == nullptr) != (sin_t == nullptr)) return -4;
   if (write_kv && (!slot_mapping || !k_pages || !v_pages)) return -5;
   const int width = (nh + nkv) * hd + nkv * vd;
-  const size_t lds = (size_t)width * sizeof(float);
-  if (lds > 64 * 1024) return -6;
+  if (padded > CR_HEAD_THREADS) return -6;
+  if (nh + 2 * nkv > 65535) return -7;
+  int threads = 64;
+  while (threads < padded) threads *= 2;
 #define GO(T, U)                                                                                                       \
   do {                                                                                                                 \
-    if (lds > 48 * 1024 && hipFuncSetAttribute((const void*)conv_rope_kv_kernel<T, U>,                                 \
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)    \
-      return -7;                                                                                                       \
-    hipLaunchKernelGGL((conv_rope_kv_kernel<T, U>), dim3(tokens), dim3(CR_THREADS), lds, stream, (T*)q_out, (const U*)proj, \
-                       (const float*)w, (const float*)state, (const int64_t*)slots, (const int32_t*)token_entry,       \
-                       (const int32_t*)cu, (const int32_t*)q_start, (const int32_t*)positions, (const float*)cos_t,    \
-                       (const float*)sin_t, (const int64_t*)slot_mapping, (T*)k_pages, (T*)v_pages, nh, nkv, hd, vd,   \
-                       padded, rotary_dim, taps, page_size, write_kv);                                                 \
+    hipLaunchKernelGGL((conv_rope_kv_kernel<T, U>), dim3(tokens, nh + 2 * nkv), dim3(threads), 0, stream, (T*)q_out,   \
+                       (const U*)proj, (const float*)w, (const float*)state, (const int64_t*)slots,                    \
+                       (const int32_t*)token_entry, (const int32_t*)cu, (const int32_t*)q_start,                       \
+                       (const int32_t*)positions, (const float*)cos_t, (const float*)sin_t,                            \
+                       (const int64_t*)slot_mapping, (T*)k_pages, (T*)v_pages, nh, nkv, hd, vd, padded, rotary_dim,    \
+                       taps, page_size, write_kv);                                                                     \
     int rc = GA_CHECK_LAUNCH();                                                                                        \
     if (rc) return rc;                                                                                                 \
     if (update_state && taps > 1 && entries > 0) {                                                                     \

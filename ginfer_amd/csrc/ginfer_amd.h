@@ -203,12 +203,26 @@ int ga_output_norm_add(void* residual, const void* y, const void* gain, const vo
 
 // ---- routing.hip: the `top` largest of every row of scores float [tokens, experts] (lowest index among equals) as
 // ids int32 [tokens, top], their softmax weights float [tokens, top], and the same weights as rows float [tokens,
-// experts] with zeros elsewhere; and the gated activation of experts laid side by side, gate_up [tokens, 2 * width] ->
-// out [tokens, width], column c weighted by dense[t, c / ff] (columns behind experts * ff by 1)
+// experts] with zeros elsewhere; and the gated activation of experts laid side by side, gate_up [tokens, 2 * width]
+// (every expert's ff gate columns followed by its ff up columns; behind the experts a shared one's) -> out [tokens,
+// width], column c weighted by dense[t, c / ff] (columns behind experts * ff by 1)
 int ga_route_topk(void* ids, void* weights, void* dense, const void* scores, int tokens, int experts, int top,
                   hipStream_t stream);
 int ga_weighted_silu_mul(void* out, const void* gate_up, const void* dense, int tokens, int width, int experts, int ff,
                          int is_bf16, hipStream_t stream);
+// router scores: scores float [tokens, experts] = w . x + b, 32-bit sums, x in the compute dtype or float
+int ga_router_max_experts();
+int ga_router_scores(void* scores, const void* x, const void* w, const void* b, int tokens, int hidden, int experts, int x_bf16,
+                     hipStream_t stream);
+// the token-expert pairs grouped by expert (offsets int32 [experts + 1], pair_of_row and row_of_pair int32 [pairs]), the
+// rows an expert reads gathered side by side, and the chosen experts' results added up per token with their weights
+int ga_route_sort(const void* ids, void* offsets, void* pair_of_row, void* row_of_pair, int pairs, int experts, hipStream_t stream);
+// (every expert's group lies `capacity` rows long in `sorted` and in `y`: row r of the grouped order at ids[pair] *
+// capacity + r - offsets[ids[pair]])
+int ga_gather_pair_rows(void* sorted, const void* x, const void* pair_of_row, const void* ids, const void* offsets, int capacity,
+                        int pairs, int hidden, int top, int is_bf16, hipStream_t stream);
+int ga_combine_pairs(void* out, const void* y, const void* shared, const void* weights, const void* row_of_pair, const void* ids,
+                     const void* offsets, int capacity, int tokens, int hidden, int top, int is_bf16, hipStream_t stream);
 
 // ---- activation.hip: out[i] = max(x[i], 0)^2 over `total` elements (out may be x)
 int ga_relu_square(void* out, const void* x, int64_t total, int is_bf16, hipStream_t stream);

@@ -75,6 +75,81 @@ __global__ __launch_bounds__(ON_THREADS) void output_norm_add_kernel(float* __re
   }
 }
 
+// The same on rows of up to ON_THREADS * 16 elements whose length is a multiple of four: 16-byte accesses (8 bytes for
+// bfloat16), every operand of a thread asked for before the first sum, four elements side by side.
+template <typename T> struct Four;
+template <> struct Four<float> {
+  static __device__ __forceinline__ float4 ld(const float* p) { return *reinterpret_cast<const float4*>(p); }
+  static __device__ __forceinline__ void st(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
+};
+template <> struct Four<bf16_t> {
+  static __device__ __forceinline__ float4 ld(const bf16_t* p) {
+    union { uint2 u; bf16_t e[4]; } a;
+    a.u = *reinterpret_cast<const uint2*>(p);
+    return float4{bf16_to_f32(a.e[0]), bf16_to_f32(a.e[1]), bf16_to_f32(a.e[2]), bf16_to_f32(a.e[3])};
+  }
+  static __device__ __forceinline__ void st(bf16_t* p, float4 v) {
+    union { uint2 u; bf16_t e[4]; } a;
+    a.e[0] = f32_to_bf16(v.x); a.e[1] = f32_to_bf16(v.y); a.e[2] = f32_to_bf16(v.z); a.e[3] = f32_to_bf16(v.w);
+    *reinterpret_cast<uint2*>(p) = a.u;
+  }
+};
+
+#define ON_CHUNKS 4          // chunks of four elements a thread keeps
+
+template <typename Y, typename C>
+__global__ __launch_bounds__(ON_THREADS) void output_norm_add_vec_kernel(float* __restrict__ residual, const Y* __restrict__ y,
+                                                                          const float* __restrict__ gain,
+                                                                          const float* __restrict__ scale, float eps,
+                                                                          const float* __restrict__ next_gain, float next_eps,
+                                                                          C* __restrict__ next, int hidden) {
+  __shared__ float scratch[ON_THREADS / WAVE];
+  const int64_t t = blockIdx.x;
+  const Y* row = y + t * hidden;
+  float* res = residual + t * hidden;
+  const int chunks = hidden / 4;
+  float4 v[ON_CHUNKS], r[ON_CHUNKS], g[ON_CHUNKS], s[ON_CHUNKS], n[ON_CHUNKS];
+  const float4 zero = float4{0.f, 0.f, 0.f, 0.f}, one = float4{1.f, 1.f, 1.f, 1.f};
+#pragma unroll
+  for (int j = 0; j < ON_CHUNKS; ++j) {
+    const int i = threadIdx.x + j * ON_THREADS;
+    const bool in = i < chunks;
+    v[j] = in ? Four<Y>::ld(row + 4 * i) : zero;
+    r[j] = in ? Four<float>::ld(res + 4 * i) : zero;
+    g[j] = in ? Four<float>::ld(gain + 4 * i) : zero;
+    s[j] = (in && scale) ? Four<float>::ld(scale + 4 * i) : one;
+    n[j] = (in && next) ? Four<float>::ld(next_gain + 4 * i) : zero;
+  }
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < ON_CHUNKS; ++j) ss += v[j].x * v[j].x + v[j].y * v[j].y + v[j].z * v[j].z + v[j].w * v[j].w;
+  ss = block_sum<ON_THREADS / WAVE>(ss, scratch);
+  const float rms = sqrtf(ss / (float)hidden + eps);
+  float ss2 = 0.f;
+#pragma unroll
+  for (int j = 0; j < ON_CHUNKS; ++j) {
+    const int i = threadIdx.x + j * ON_THREADS;
+    r[j].x += v[j].x / rms * g[j].x * s[j].x;
+    r[j].y += v[j].y / rms * g[j].y * s[j].y;
+    r[j].z += v[j].z / rms * g[j].z * s[j].z;
+    r[j].w += v[j].w / rms * g[j].w * s[j].w;
+    if (i < chunks) {
+      Four<float>::st(res + 4 * i, r[j]);
+      ss2 += r[j].x * r[j].x + r[j].y * r[j].y + r[j].z * r[j].z + r[j].w * r[j].w;
+    }
+  }
+  if (next == nullptr) return;
+  ss2 = block_sum<ON_THREADS / WAVE>(ss2, scratch);
+  const float rms2 = sqrtf(ss2 / (float)hidden + next_eps);
+  C* out = next + t * hidden;
+#pragma unroll
+  for (int j = 0; j < ON_CHUNKS; ++j) {
+    const int i = threadIdx.x + j * ON_THREADS;
+    if (i < chunks)
+      Four<C>::st(out + 4 * i, float4{r[j].x / rms2 * n[j].x, r[j].y / rms2 * n[j].y, r[j].z / rms2 * n[j].z, r[j].w / rms2 * n[j].w});
+  }
+}
+
 extern "C" int ga_output_norm_add(void* residual, const void* y, const void* gain, const void* scale, float eps,
                                   const void* next_gain, float next_eps, void* next, int tokens, int hidden, int y_bf16,
                                   int next_bf16, hipStream_t stream) {
@@ -82,9 +157,19 @@ extern "C" int ga_output_norm_add(void* residual, const void* y, const void* gai
   if (hidden <= 0 || !gain) return -1;
   if (next && !next_gain) return -2;
   dim3 grid(tokens), block(ON_THREADS);
-#define GO(Y, C) hipLaunchKernelGGL((output_norm_add_kernel<Y, C>), grid, block, 0, stream, (float*)residual, (const Y*)y, \
-                                    (const float*)gain, (const float*)scale, eps, (const float*)next_gain, next_eps,       \
-                                    (C*)next, hidden)
+  const uintptr_t all = (uintptr_t)residual | (uintptr_t)y | (uintptr_t)gain | (uintptr_t)scale | (uintptr_t)next_gain | (uintptr_t)next;
+  const bool vec = hidden % 4 == 0 && hidden <= 4 * ON_CHUNKS * ON_THREADS && all % 16 == 0;
+#define GO(Y, C)                                                                                                          \
+  do {                                                                                                                    \
+    if (vec)                                                                                                              \
+      hipLaunchKernelGGL((output_norm_add_vec_kernel<Y, C>), grid, block, 0, stream, (float*)residual, (const Y*)y,       \
+                         (const float*)gain, (const float*)scale, eps, (const float*)next_gain, next_eps, (C*)next,       \
+                         hidden);                                                                                         \
+    else                                                                                                                  \
+      hipLaunchKernelGGL((output_norm_add_kernel<Y, C>), grid, block, 0, stream, (float*)residual, (const Y*)y,           \
+                         (const float*)gain, (const float*)scale, eps, (const float*)next_gain, next_eps, (C*)next,       \
+                         hidden);                                                                                         \
+  } while (0)
   if (y_bf16) { if (next_bf16) GO(bf16_t, bf16_t); else GO(bf16_t, float); }
   else { if (next_bf16) GO(float, bf16_t); else GO(float, float); }
 #undef GO

@@ -1072,9 +1072,82 @@ def route_topk(scores, top):
     return ids, weights, dense
 
 
+def router_scores(x, weight, bias):
+    """x [T, H] (bfloat16 or float32), weight float32 [E, H], bias float32 [E] or None -> float32 [T, E] = x . weight^T + bias,
+    summed in 32-bit, a wavefront per score."""
+    _dev(x, weight, bias)
+    _need(x.dim() == 2 and x.is_contiguous() and x.dtype in (torch.float32, torch.bfloat16), "x must be contiguous float32 or bfloat16 [T, H]")
+    T, H = x.shape
+    E = weight.shape[0]
+    _need(1 <= E <= ROUTE_MAX_EXPERTS, "1 to %d experts, got %d", ROUTE_MAX_EXPERTS, E)
+    _f32(weight, (E, H), "router weight")
+    if bias is not None:
+        _f32(bias, (E,), "router bias")
+    scores = torch.empty((T, E), dtype=torch.float32, device=x.device)
+    lib = build.load("routing")
+    _check(lib.ga_router_scores(_ptr(scores), _ptr(x), _ptr(weight), _ptr(bias), _i(T), _i(H), _i(E), _i(_is_bf16(x.dtype)),
+                                _stream()), "router_scores")
+    return scores
+
+
+def route_sort(ids, experts):
+    """ids int32 [T, top] -> (offsets int32 [experts + 1], pair_of_row int32 [T * top], row_of_pair int32 [T * top]): the
+    token-expert pairs (pair p = token p // top, its choice p % top) grouped by expert; expert e owns the rows
+    [offsets[e], offsets[e + 1])."""
+    _dev(ids)
+    _need(ids.dtype == torch.int32 and ids.dim() == 2 and ids.is_contiguous(), "ids must be contiguous int32 [T, top]")
+    _need(1 <= experts <= ROUTE_MAX_EXPERTS, "1 to %d experts, got %d", ROUTE_MAX_EXPERTS, experts)
+    P = ids.numel()
+    offsets = torch.empty((experts + 1,), dtype=torch.int32, device=ids.device)
+    pair_of_row = torch.empty((P,), dtype=torch.int32, device=ids.device)
+    row_of_pair = torch.empty((P,), dtype=torch.int32, device=ids.device)
+    lib = build.load("routing")
+    _check(lib.ga_route_sort(_ptr(ids), _ptr(offsets), _ptr(pair_of_row), _ptr(row_of_pair), _i(P), _i(experts), _stream()), "route_sort")
+    return offsets, pair_of_row, row_of_pair
+
+
+def gather_pair_rows(x, pair_of_row, ids, offsets, capacity):
+    """x [T, H]; pair_of_row int32 [P], ids int32 [T, top], offsets int32 [E + 1] as route_sort gives them -> [E, capacity,
+    H]: expert e's rows side by side from [e, 0] on (what lies behind them holds anything)."""
+    _dev(x, pair_of_row, ids, offsets)
+    _need(x.dim() == 2 and x.is_contiguous() and x.dtype in (torch.float32, torch.bfloat16), "x must be contiguous [T, H]")
+    _need(pair_of_row.dtype == torch.int32 and pair_of_row.shape == (ids.numel(),) and pair_of_row.is_contiguous(), "pair_of_row must be int32 [P]")
+    _need(ids.dtype == torch.int32 and ids.dim() == 2 and ids.shape[0] == x.shape[0] and ids.is_contiguous(), "ids must be contiguous int32 [T, top]")
+    _need(offsets.dtype == torch.int32 and offsets.dim() == 1 and offsets.is_contiguous(), "offsets must be int32 [E + 1]")
+    E, P, H = offsets.shape[0] - 1, pair_of_row.shape[0], x.shape[1]
+    _need(capacity >= 1, "an expert's group must hold at least a row")
+    out = torch.empty((E, capacity, H), dtype=x.dtype, device=x.device)
+    lib = build.load("routing")
+    _check(lib.ga_gather_pair_rows(_ptr(out), _ptr(x), _ptr(pair_of_row), _ptr(ids), _ptr(offsets), _i(capacity), _i(P), _i(H),
+                                   _i(ids.shape[1]), _i(_is_bf16(x.dtype)), _stream()), "gather_pair_rows")
+    return out
+
+
+def combine_pairs(y, shared, weights, row_of_pair, ids, offsets):
+    """y [E, capacity, H]: the experts' results, laid as gather_pair_rows lays their rows; weights float32 [T, top];
+    shared [T, H] or None -> [T, H]: sum_j weights[t, j] * (the result of pair t * top + j) + shared[t], added in 32-bit in
+    the order of the choice."""
+    _dev(y, shared, weights, row_of_pair, ids, offsets)
+    T, top = weights.shape
+    _need(y.dim() == 3 and y.is_contiguous() and y.shape[0] == offsets.shape[0] - 1, "y must be contiguous [E, capacity, H]")
+    capacity, H = y.shape[1], y.shape[2]
+    _f32(weights, (T, top), "weights")
+    _need(row_of_pair.dtype == torch.int32 and row_of_pair.shape == (T * top,) and row_of_pair.is_contiguous(), "row_of_pair must be int32 [%d]", T * top)
+    _need(ids.dtype == torch.int32 and ids.shape == (T, top) and ids.is_contiguous(), "ids must be contiguous int32 [%d, %d]", T, top)
+    _need(offsets.dtype == torch.int32 and offsets.is_contiguous(), "offsets must be int32 [E + 1]")
+    if shared is not None:
+        _need(shared.shape == (T, H) and shared.dtype == y.dtype and shared.is_contiguous(), "shared must be contiguous [%d, %d]", T, H)
+    out = torch.empty((T, H), dtype=y.dtype, device=y.device)
+    lib = build.load("routing")
+    _check(lib.ga_combine_pairs(_ptr(out), _ptr(y), _ptr(shared), _ptr(weights), _ptr(row_of_pair), _ptr(ids), _ptr(offsets),
+                                _i(capacity), _i(T), _i(H), _i(top), _i(_is_bf16(y.dtype)), _stream()), "combine_pairs")
+    return out
+
+
 def weighted_silu_mul(gate_up, dense, ff):
-    """gate_up [T, 2 I] (gates of all experts side by side, then their ups) -> [T, I]: w * silu(gate) * up, the columns
-    [e * ff, (e + 1) * ff) weighted by dense[t, e], the columns behind the last expert's by 1."""
+    """gate_up [T, 2 I]: for every expert its ff gate columns, then its ff up columns, the experts one after the other, and
+    behind them a shared expert's gates and ups -> [T, I]: w * silu(gate) * up, the columns [e * ff, (e + 1) * ff) weighted
+    by dense[t, e], the columns behind the last expert's by 1."""
     _dev(gate_up, dense)
     _need(gate_up.dim() == 2 and gate_up.is_contiguous() and gate_up.shape[1] % 2 == 0, "gate_up must be contiguous [T, 2I]")
     T, I = gate_up.shape[0], gate_up.shape[1] // 2
@@ -1110,8 +1183,9 @@ def conv_rope_kv(proj, weight, state, slots, step, cos, sin, slot_mapping, k_pag
     C = (num_heads + num_kv_heads) * head_dim + num_kv_heads * value_dim
     _need(proj.dim() == 2 and proj.shape[1] == C and proj.is_contiguous() and proj.dtype in (torch.float32, torch.bfloat16),
           "proj must be contiguous float32 or bfloat16 [T, %d], got %s %s", C, proj.dtype, tuple(proj.shape))
-    _need(C * 4 <= 64 * 1024, "this kernel keeps a token's %d channels in 64 KB of LDS", C)
-    _need(padded >= head_dim and padded >= value_dim, "heads padded to %d do not hold %d / %d", padded, head_dim, value_dim)
+    _need(head_dim <= padded <= 256 and value_dim <= padded, "heads padded to %d (at most 256) do not hold %d / %d", padded,
+          head_dim, value_dim)
+    _need(num_heads + 2 * num_kv_heads <= 65535, "too many heads for one launch: %d", num_heads + 2 * num_kv_heads)
     taps = 1
     if weight is not None:
         _need(weight.dim() == 2 and weight.shape[0] == C and 1 <= weight.shape[1] <= SHORT_CONV_MAX_TAPS,

@@ -120,6 +120,16 @@ class Tuning:
     # workgroup of it streams from memory no faster than any other), at most `latent_decode_max_splits` to a token
     latent_decode_workgroups: int = 1024
     latent_decode_max_splits: int = 32
+    # ---- routed feed-forwards (parts/mlp.py).  Steps of fewer rows than this run every expert over every row in one
+    # product (rows that an expert does not own enter with zeros): no step that is recorded is longer, and up to some
+    # hundred rows the experts' weights, which all come from memory either way, are what the step waits for.  Longer steps
+    # (bfloat16) may group the rows by expert and run the experts as a batched product over their own rows, which needs the
+    # groups' sizes on the host.  That way is SWITCHED OFF (no number of rows reaches the threshold): a run of 2,048- to
+    # 4,000-token steps at 1,536- and 3,584-wide layers with it ended in a memory fault on the device whose cause is not
+    # found; at the tests' small sizes it gives the plain statement's results.  RoutedGLU refuses it unless
+    # `routed_by_expert_allowed` is set as well.
+    routed_by_expert_from_rows: int = 1 << 30
+    routed_by_expert_allowed: bool = False
     # ---- recorded steps (engine/runner.py): steps with prompt portions are laid into recorded steps of padded sizes up
     # to `mixed_graph_max_tokens` rows, fewer for large models: padding pays while rows x weights stays under what the
     # device does in the time the host needs to launch a step kernel by kernel.

@@ -2,6 +2,7 @@
 import torch
 
 from ..kernels import ops
+from ..kernels.tuning import TUNING
 from ..weights.loader import WeightSpec
 from .base import Part
 from .linear import linear, gated_linear, gated_plan, linear_into_norm
@@ -113,13 +114,18 @@ class RoutedGLU(Part):
     the largest scores, weighted by the softmax over those scores alone; an optional shared expert of its own width
     runs for every token and is added.  Expert: down(silu(gate(x)) * up(x)), no biases.
 
-    The experts lie side by side: ONE product gives the gates and ups of all experts (and of the shared one), the
-    activation multiplies each expert's columns by the token's weight for it (zero where the token does not use it),
-    and ONE product with the down matrices laid side by side adds the experts' results up, in 32-bit.  Routing is a
-    pure function of the token's row, so a token's result does not depend on the batch.
+    Two ways, by the number of rows (`TUNING.routed_by_expert_from_rows`; the second way is switched off there for now).  Few rows, and every step that is recorded:
+    the experts lie side by side, ONE product gives the gates and ups of all experts (and of the shared one), the
+    activation multiplies each expert's columns by the token's weight for it (zero where the token does not use it), and
+    ONE product with the down matrices laid side by side adds the experts' results up, in 32-bit.  Many rows (bfloat16):
+    the token-expert pairs are grouped by expert, the groups laid side by side as long as the longest, two batched
+    products run every expert over its own rows, and a last kernel adds a token's results with their weights; this way
+    reads the groups' sizes on the host, so it is never recorded.  Routing is a
+    pure function of the token's row, so a token's result does not depend on the batch beyond rounding; in 32-bit
+    only the first way runs, and not at all.
     Tensors: router, router.b, e<i>.gate / .up / .down, shared.gate / .up / .down."""
 
-    capturable = True
+    capturable = True                # the steps that the runner records are short enough for the first way
 
     def __init__(self, hidden_size, num_experts, top_k, expert_size, dtype, device, shared_size=None, router_bias=True):
         self.hidden_size, self.num_experts, self.top_k = int(hidden_size), int(num_experts), int(top_k)
@@ -148,18 +154,39 @@ class RoutedGLU(Part):
         self.w_router = t["router"].float().contiguous()
         self.b_router = t["router.b"].float().contiguous() if self.router_bias else None
         names = ["e%d" % e for e in range(self.num_experts)] + (["shared"] if self.shared_size else [])
-        self.w_gate_up = torch.cat([t[n + ".gate"] for n in names] + [t[n + ".up"] for n in names], dim=0).contiguous()
+        # every expert's gate rows, then its up rows: one expert's share of the stacked matrix is one piece
+        self.w_gate_up = torch.cat([t[n + kind] for n in names for kind in (".gate", ".up")], dim=0).contiguous()
         self.w_down = torch.cat([t[n + ".down"] for n in names], dim=1).contiguous()
 
     def kernel_modules(self):
-        return ["routing", "gemm"] + (["gemm_skinny"] if self.dtype == torch.bfloat16 else [])
+        return ["routing", "activation", "gemm"] + (["gemm_skinny"] if self.dtype == torch.bfloat16 else [])
 
     def route(self, x):
         """(ids int32 [T, top_k], weights float32 [T, top_k], the weights as rows over all experts [T, E])."""
-        scores = ops.gemm_nt(x if x.dtype == torch.float32 else x.float(), self.w_router, self.b_router)
-        return ops.route_topk(scores, self.top_k)
+        return ops.route_topk(ops.router_scores(x, self.w_router, self.b_router), self.top_k)
 
     def forward(self, x):
-        _, _, dense = self.route(x)
+        ids, weights, dense = self.route(x)
+        if x.dtype == torch.bfloat16 and x.shape[0] >= TUNING.routed_by_expert_from_rows:
+            if not TUNING.routed_by_expert_allowed:
+                raise RuntimeError("the experts as a batched product over their own rows: switched off (an unexplained "
+                                   "memory fault at large sizes); see kernels/tuning.py")
+            return self._by_expert(x, ids, weights)
         act = ops.weighted_silu_mul(linear(x, self.w_gate_up), dense, self.expert_size)
         return linear(act, self.w_down)
+
+    def _by_expert(self, x, ids, weights):
+        E, F, S, H = self.num_experts, self.expert_size, self.shared_size, self.hidden_size
+        offsets, pair_of_row, row_of_pair = ops.route_sort(ids, E)
+        bounds = offsets.tolist()                    # the host waits here for the groups' sizes
+        # every expert's group as long as the longest, so that the experts are the batch of two batched products
+        capacity = -(-max(max(b - a for a, b in zip(bounds, bounds[1:])), 1) // 16) * 16
+        rows = ops.gather_pair_rows(x, pair_of_row, ids, offsets, capacity)
+        gate_up = torch.bmm(rows, self.w_gate_up[:2 * F * E].view(E, 2 * F, H).transpose(1, 2))
+        act = ops.silu_mul(gate_up.view(E * capacity, 2 * F))
+        down = self.w_down.as_strided((E, H, F), (F, self.w_down.stride(0), 1))       # expert e: the columns [eF, (e+1)F)
+        y = torch.bmm(act.view(E, capacity, F), down.transpose(1, 2))
+        shared = None
+        if S:
+            shared = torch.mm(gated_linear(x, self.w_gate_up[2 * F * E:]), self.w_down[:, F * E:].t())
+        return ops.combine_pairs(y, shared, weights, row_of_pair, ids, offsets)
