@@ -196,10 +196,11 @@ int ga_conv_rope_kv(void* q_out, const void* proj, const void* w, void* state, c
 
 // ---- output_norm.hip: residual[t] += scale * gain * y[t] / sqrt(mean(y[t]^2) + eps) (a norm on a sublayer's output, a
 // factor per channel behind it; gain and scale float [hidden], scale may be null); with `next` also next[t] = next_gain *
-// residual[t] / sqrt(mean(residual[t]^2) + next_eps), the rows that the following sublayer reads, in the compute dtype
+// residual[t] / sqrt(mean(residual[t]^2) + next_eps), the rows that the following sublayer reads, in the compute dtype;
+// parts > 1: y is float [parts, tokens, hidden], partial sums that are added in order first
 int ga_output_norm_add(void* residual, const void* y, const void* gain, const void* scale, float eps,
                        const void* next_gain, float next_eps, void* next, int tokens, int hidden, int y_bf16,
-                       int next_bf16, hipStream_t stream);
+                       int next_bf16, int parts, hipStream_t stream);
 
 // ---- routing.hip: the `top` largest of every row of scores float [tokens, experts] (lowest index among equals) as
 // ids int32 [tokens, top], their softmax weights float [tokens, top], and the same weights as rows float [tokens,

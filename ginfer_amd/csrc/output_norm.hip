@@ -1,6 +1,7 @@
 // A norm on a sublayer's OUTPUT with a factor per channel behind it, fused with the residual add and, where the caller
 // wants it, with the norm that the NEXT sublayer reads through:
 //   residual[t] += s * g * y[t] / sqrt(mean(y[t]^2) + eps)                  g, s: one number per channel (s may be absent)
+//   (y may come as the 32-bit partial sums [parts, tokens, hidden] of a product whose K was split: added in order first)
 //   next[t]      = g2 * residual[t] / sqrt(mean(residual[t]^2) + eps2)      (optional; in the compute dtype)
 // The row stays in registers between the two (up to ON_THREADS * ON_PER elements; longer rows are read again).
 // All arithmetic in 32-bit; a row's sums are taken in an order that depends on its length alone.
@@ -15,24 +16,31 @@ __global__ __launch_bounds__(ON_THREADS) void output_norm_add_kernel(float* __re
                                                                       const float* __restrict__ gain,
                                                                       const float* __restrict__ scale, float eps,
                                                                       const float* __restrict__ next_gain, float next_eps,
-                                                                      C* __restrict__ next, int hidden) {
+                                                                      C* __restrict__ next, int hidden, int parts,
+                                                                      int64_t part_stride) {
   __shared__ float scratch[ON_THREADS / WAVE];
   const int64_t t = blockIdx.x;
   const Y* row = y + t * hidden;
   float* res = residual + t * hidden;
   const bool kept = hidden <= ON_THREADS * ON_PER;
+  // y may be the partial sums of a product whose K was split (parts > 1, 32-bit): they are added in order
+  auto value = [&](int i) {
+    float a = Num<Y>::ld(row + i);
+    for (int p = 1; p < parts; ++p) a += Num<Y>::ld(row + p * part_stride + i);
+    return a;
+  };
   float v[ON_PER];
   float ss = 0.f;
   if (kept) {
 #pragma unroll
     for (int j = 0; j < ON_PER; ++j) {
       const int i = threadIdx.x + j * ON_THREADS;
-      v[j] = i < hidden ? Num<Y>::ld(row + i) : 0.f;
+      v[j] = i < hidden ? value(i) : 0.f;
       ss += v[j] * v[j];
     }
   } else {
     for (int i = threadIdx.x; i < hidden; i += ON_THREADS) {
-      const float a = Num<Y>::ld(row + i);
+      const float a = value(i);
       ss += a * a;
     }
   }
@@ -53,7 +61,7 @@ __global__ __launch_bounds__(ON_THREADS) void output_norm_add_kernel(float* __re
     }
   } else {
     for (int i = threadIdx.x; i < hidden; i += ON_THREADS) {
-      float a = Num<Y>::ld(row + i) / rms * gain[i];
+      float a = value(i) / rms * gain[i];
       if (scale) a *= scale[i];
       const float h = res[i] + a;
       res[i] = h;
@@ -102,7 +110,8 @@ __global__ __launch_bounds__(ON_THREADS) void output_norm_add_vec_kernel(float* 
                                                                           const float* __restrict__ gain,
                                                                           const float* __restrict__ scale, float eps,
                                                                           const float* __restrict__ next_gain, float next_eps,
-                                                                          C* __restrict__ next, int hidden) {
+                                                                          C* __restrict__ next, int hidden, int parts,
+                                                                          int64_t part_stride) {
   __shared__ float scratch[ON_THREADS / WAVE];
   const int64_t t = blockIdx.x;
   const Y* row = y + t * hidden;
@@ -115,6 +124,12 @@ __global__ __launch_bounds__(ON_THREADS) void output_norm_add_vec_kernel(float* 
     const int i = threadIdx.x + j * ON_THREADS;
     const bool in = i < chunks;
     v[j] = in ? Four<Y>::ld(row + 4 * i) : zero;
+    for (int p = 1; p < parts; ++p) {              // partial sums of a product whose K was split: added in order
+      if (in) {
+        const float4 more = Four<Y>::ld(row + p * part_stride + 4 * i);
+        v[j].x += more.x; v[j].y += more.y; v[j].z += more.z; v[j].w += more.w;
+      }
+    }
     r[j] = in ? Four<float>::ld(res + 4 * i) : zero;
     g[j] = in ? Four<float>::ld(gain + 4 * i) : zero;
     s[j] = (in && scale) ? Four<float>::ld(scale + 4 * i) : one;
@@ -152,10 +167,12 @@ __global__ __launch_bounds__(ON_THREADS) void output_norm_add_vec_kernel(float* 
 
 extern "C" int ga_output_norm_add(void* residual, const void* y, const void* gain, const void* scale, float eps,
                                   const void* next_gain, float next_eps, void* next, int tokens, int hidden, int y_bf16,
-                                  int next_bf16, hipStream_t stream) {
+                                  int next_bf16, int parts, hipStream_t stream) {
   if (tokens <= 0) return 0;
   if (hidden <= 0 || !gain) return -1;
   if (next && !next_gain) return -2;
+  if (parts < 1 || (parts > 1 && y_bf16)) return -3;       // parts: 32-bit [parts, tokens, hidden]
+  const int64_t part_stride = (int64_t)tokens * hidden;
   dim3 grid(tokens), block(ON_THREADS);
   const uintptr_t all = (uintptr_t)residual | (uintptr_t)y | (uintptr_t)gain | (uintptr_t)scale | (uintptr_t)next_gain | (uintptr_t)next;
   const bool vec = hidden % 4 == 0 && hidden <= 4 * ON_CHUNKS * ON_THREADS && all % 16 == 0;
@@ -164,11 +181,11 @@ extern "C" int ga_output_norm_add(void* residual, const void* y, const void* gai
     if (vec)                                                                                                              \
       hipLaunchKernelGGL((output_norm_add_vec_kernel<Y, C>), grid, block, 0, stream, (float*)residual, (const Y*)y,       \
                          (const float*)gain, (const float*)scale, eps, (const float*)next_gain, next_eps, (C*)next,       \
-                         hidden);                                                                                         \
+                         hidden, parts, part_stride);                                                                     \
     else                                                                                                                  \
       hipLaunchKernelGGL((output_norm_add_kernel<Y, C>), grid, block, 0, stream, (float*)residual, (const Y*)y,           \
                          (const float*)gain, (const float*)scale, eps, (const float*)next_gain, next_eps, (C*)next,       \
-                         hidden);                                                                                         \
+                         hidden, parts, part_stride);                                                                     \
   } while (0)
   if (y_bf16) { if (next_bf16) GO(bf16_t, bf16_t); else GO(bf16_t, float); }
   else { if (next_bf16) GO(float, bf16_t); else GO(float, float); }

@@ -1028,14 +1028,22 @@ def latent_attention(qa, c_pages, block_table, step, sink, gate, heads, rank, pa
 # norm on a sublayer's output with a factor per channel, routing to experts, activations of feed-forwards without a gate
 
 def output_norm_add(residual, y, gain, scale, eps, next_gain=None, next_eps=None, dtype=None):
-    """residual float32 [T, H] += scale * gain * y / sqrt(mean(y^2) + eps), in place; y [T, H] float32 or bfloat16; gain
-    float32 [H]; scale float32 [H] or None.  With next_gain (float32 [H]) the rows next_gain * r / sqrt(mean(r^2) +
+    """residual float32 [T, H] += scale * gain * y / sqrt(mean(y^2) + eps), in place; y [T, H] float32 or bfloat16, or
+    float32 [parts, T, H]: partial sums of a product whose K was split, added in order first; gain float32 [H]; scale
+    float32 [H] or None.  With next_gain (float32 [H]) the rows next_gain * r / sqrt(mean(r^2) +
     next_eps) of the new residual r come back in `dtype`: what the sublayer after this one reads."""
     _dev(residual, y, gain, scale, next_gain)
     _need(residual.dtype == torch.float32 and residual.dim() == 2 and residual.is_contiguous(),
           "residual must be contiguous float32 [T, H]")
-    _need(y.shape == residual.shape and y.is_contiguous() and y.dtype in (torch.float32, torch.bfloat16),
-          "y must be contiguous float32 or bfloat16 %s, got %s %s", tuple(residual.shape), y.dtype, tuple(y.shape))
+    parts = 1
+    if y.dim() == 3:
+        _need(y.dtype == torch.float32 and tuple(y.shape[1:]) == tuple(residual.shape) and y.is_contiguous() and y.shape[0] >= 1,
+              "partial sums must be contiguous float32 [parts, %d, %d], got %s %s", residual.shape[0], residual.shape[1], y.dtype,
+              tuple(y.shape))
+        parts = y.shape[0]
+    else:
+        _need(y.shape == residual.shape and y.is_contiguous() and y.dtype in (torch.float32, torch.bfloat16),
+              "y must be contiguous float32 or bfloat16 %s, got %s %s", tuple(residual.shape), y.dtype, tuple(y.shape))
     T, H = residual.shape
     _f32(gain, (H,), "gain")
     if scale is not None:
@@ -1048,7 +1056,7 @@ def output_norm_add(residual, y, gain, scale, eps, next_gain=None, next_eps=None
     lib = build.load("output_norm")
     _check(lib.ga_output_norm_add(_ptr(residual), _ptr(y), _ptr(gain), _ptr(scale), _f(eps), _ptr(next_gain),
                                   _f(next_eps if next_eps is not None else 0.0), _ptr(out), _i(T), _i(H), _i(_is_bf16(y.dtype)),
-                                  _i(_is_bf16(dtype)) if out is not None else _i(0), _stream()), "output_norm_add")
+                                  _i(_is_bf16(dtype)) if out is not None else _i(0), _i(parts), _stream()), "output_norm_add")
     return out
 
 

@@ -104,4 +104,4 @@ class ConvAttention(Part):
                              update_state=state is not None and state.owner)
         a = ops.paged_attention(q, kv.k_pages, kv.v_pages, kv.block_table, step, self.nh, self.nkv, self.padded,
                                 self.scale, self.window, sinks=self.sinks)
-        return linear(a, self.w_o, None)
+        return linear(a, self.w_o, None, parts_ok=True)

@@ -105,7 +105,8 @@ class SquaredReLU(Part):
         return ["activation", "gemm"] + (["gemm_skinny"] if self.dtype == torch.bfloat16 else [])
 
     def forward(self, x):
-        return linear(ops.relu_square(linear(x, self.w_up)), self.w_down)
+        # the result may be partial sums of a K-split product: the norm that follows adds them up
+        return linear(ops.relu_square(linear(x, self.w_up)), self.w_down, parts_ok=True)
 
 
 @register_feed_forward("routed_glu")
@@ -173,7 +174,7 @@ class RoutedGLU(Part):
                                    "memory fault at large sizes); see kernels/tuning.py")
             return self._by_expert(x, ids, weights)
         act = ops.weighted_silu_mul(linear(x, self.w_gate_up), dense, self.expert_size)
-        return linear(act, self.w_down)
+        return linear(act, self.w_down, parts_ok=True)     # maybe partial sums: the norm that follows adds them up
 
     def _by_expert(self, x, ids, weights):
         E, F, S, H = self.num_experts, self.expert_size, self.shared_size, self.hidden_size

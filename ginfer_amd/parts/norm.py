@@ -49,7 +49,7 @@ class ScaledOutputRMSNorm(Part):
     inside the part (scale_name None: no such factor)."""
 
     capturable = True
-    accepts_partial_sums = False
+    accepts_partial_sums = True      # add_normed takes float32 [parts, T, H] and adds the parts up in order
     foldable = False
 
     def __init__(self, size, eps, dtype, device, gain_offset=0.0, gain_name="weight", scale_name="scale"):
@@ -73,8 +73,6 @@ class ScaledOutputRMSNorm(Part):
         return ["output_norm"]
 
     def add_normed(self, residual, y, then=None):
-        if y.dim() == 3:                         # partial sums of a product whose K was split
-            y = y.sum(dim=0)
         if then is None:
             return ops.output_norm_add(residual, y, self.weight, self.scale, self.eps)
         gain = then.weight if then.weight.dtype == torch.float32 else then.weight.float()

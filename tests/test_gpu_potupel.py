@@ -193,6 +193,13 @@ def test_output_norm_with_layer_scale_and_the_next_norm():
                 r2 = res.cuda().clone()
                 assert ops.output_norm_add(r2, yy.cuda(), gain.cuda(), scale.cuda() if with_scale else None, 1e-5) is None
                 assert torch.equal(r2, r)
+        # the sublayer's result as three partial sums of a product whose K was split
+        parts = torch.randn((3, 5, width), generator=g) * 0.1
+        r = res.cuda().clone()
+        rows = ops.output_norm_add(r, parts.cuda(), gain.cuda(), scale.cuda(), 1e-5, nxt.cuda(), 3e-6, torch.float32)
+        whole = (parts[0] + parts[1]) + parts[2]
+        want = res.double() + pp.centered_norm(whole.double(), gain.double() - 1.0, 1e-5) * scale.double()
+        assert H.rel_err(r.cpu(), want) < 2e-6 and H.rel_err(rows.cpu(), pp.centered_norm(want, nxt.double() - 1.0, 3e-6)) < 2e-6
 
 
 def test_norm_with_a_gain_stored_around_zero():
