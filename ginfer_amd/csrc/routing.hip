@@ -133,9 +133,20 @@ __global__ __launch_bounds__(256) void router_scores_kernel(float* __restrict__ 
   const int e = (int)(p - t * experts);
   const T* row = x + t * hidden;
   const float* we = w + (int64_t)e * hidden;
-  float acc = 0.f;
-  for (int k = lane; k < hidden; k += WAVE) acc += we[k] * Num<T>::ld(row + k);
-  acc = wave_sum(acc);
+  // four sums a lane, so that four pairs of loads are under way at a time; added in a fixed order
+  float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+  int k = lane;
+  for (; k + 3 * WAVE < hidden; k += 4 * WAVE) {
+    const float w0 = we[k], w1 = we[k + WAVE], w2 = we[k + 2 * WAVE], w3 = we[k + 3 * WAVE];
+    const float x0 = Num<T>::ld(row + k), x1 = Num<T>::ld(row + k + WAVE), x2 = Num<T>::ld(row + k + 2 * WAVE),
+                x3 = Num<T>::ld(row + k + 3 * WAVE);
+    a0 += w0 * x0;
+    a1 += w1 * x1;
+    a2 += w2 * x2;
+    a3 += w3 * x3;
+  }
+  for (; k < hidden; k += WAVE) a0 += we[k] * Num<T>::ld(row + k);
+  float acc = wave_sum((a0 + a1) + (a2 + a3));
   if (lane == 0) scores[p] = acc + (b ? b[e] : 0.f);
 }
 
