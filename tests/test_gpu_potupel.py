@@ -218,7 +218,7 @@ def test_norm_with_a_gain_stored_around_zero():
 def test_routing_chooses_the_largest_and_weighs_them_alone():
     from ginfer_amd.kernels import ops
     g = torch.Generator().manual_seed(2)
-    for experts, top in ((8, 3), (5, 5), (3, 1), (70, 6), (256, 9), (1, 1)):
+    for experts, top in ((10, 3), (5, 5), (3, 1), (70, 6), (256, 9), (1, 1)):
         z = torch.randn((37, experts), generator=g) * 2
         z[3] = 0.25                                   # all equal: the lowest indices win
         if experts > 2:
@@ -236,7 +236,7 @@ def test_routing_chooses_the_largest_and_weighs_them_alone():
 def test_router_scores_in_32_bit():
     from ginfer_amd.kernels import ops
     g = torch.Generator().manual_seed(8)
-    for experts, hidden, tokens in ((8, 320, 37), (1, 40, 3), (32, 100, 5), (70, 64, 9), (256, 130, 2)):
+    for experts, hidden, tokens in ((6, 272, 37), (1, 40, 3), (32, 100, 5), (70, 64, 9), (256, 130, 2)):
         x = torch.randn((tokens, hidden), generator=g)
         w, b = torch.randn((experts, hidden), generator=g), torch.randn((experts,), generator=g)
         for dtype in (torch.float32, torch.bfloat16):
@@ -386,7 +386,7 @@ def _sink_case(seqs, nh, nkv, hd, ps, dtype, seed, scale, spike=None, sink_score
 
 
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.bfloat16, 2e-2)])
-@pytest.mark.parametrize("nh,nkv,hd", [(8, 1, 64), (6, 3, 16), (4, 4, 48), (3, 1, 128), (5, 5, 40)])
+@pytest.mark.parametrize("nh,nkv,hd", [(6, 1, 64), (6, 3, 16), (4, 4, 48), (3, 1, 128), (5, 5, 40)])
 @pytest.mark.parametrize("seqs", [[(1, 1), (1, 2), (2, 2), (1, 17), (33, 40)], [(1, 300), (20, 300), (1, 64), (1, 65)],
                                   [(125, 260), (63, 63)], [(1, 1500)], [(300, 700)]])
 def test_attention_with_a_sink_in_every_kernel(dtype, tol, nh, nkv, hd, seqs):
