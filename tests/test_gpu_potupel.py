@@ -87,12 +87,12 @@ def make_folder(path, cfg, seed, std_scale=5.0, edit=None):
 
 
 def sharpen(tensors):
-    """Convolutions of moderate size, and queries large enough that one key takes most of a softmax in many rows (a key
+    """Convolutions of moderate size whatever their number of taps, and queries large enough that one key takes most of a softmax in many rows (a key
     that is wrongly seen or missed then moves the result) while other rows keep scores near zero, where the sink holds
     a visible share; routers with wide margins, so that few choices are close calls."""
     for name, t in tensors.items():
         if name.endswith(".conv"):
-            t *= 0.25
+            t *= 0.4 / t.shape[1] ** 0.5              # a channel's taps together about as large as one tap of 1
         if name.endswith(".mix.q"):
             t *= 2.0
         if name.endswith(".router") or name.endswith(".router.b"):
@@ -126,20 +126,22 @@ def plain(folder, ids):
     return _plain[key]
 
 
-def compare(got, requests, folder, tol, what, close_calls=0.0):
+def compare(got, requests, folder, tol, what, close_calls=0.0, median=0.5):
     """Every row against the plain statement.  close_calls: the share of rows that may miss the tolerance (bfloat16:
     where two experts' scores lie within rounding of each other the engine may choose the other one; that row, and
     faintly the rows that attend to it, then differ by more than rounding)."""
-    over, first = 0, None
+    over, first, errors = 0, None, []
     for (rid, p), row in sorted(got.items()):
         ref = plain(folder, requests[rid])
         assert np.isfinite(row).all(), "%s: request %s position %d: non-finite logits" % (what, rid, p)
         err = float(np.abs(row.astype(np.float64) - ref[p]).max() / np.abs(ref).max())
+        errors.append(err)
         if err > tol:
             over += 1
             first = first or "%s: first wrong place is request %s position %d of %d: error %.3g > %.3g" % (
                 what, rid, p, len(requests[rid]), err, tol)
     assert over <= close_calls * len(got), "%s (%d of %d rows)" % (first, over, len(got))
+    assert float(np.median(errors)) <= tol * median, "%s: the median row is off by %.3g" % (what, float(np.median(errors)))
     for rid, ids in requests.items():
         missing = [p for p in range(len(ids)) if (rid, p) not in got]
         assert not missing, "%s: request %s lacks logits at %s" % (what, rid, missing[:8])
@@ -147,9 +149,12 @@ def compare(got, requests, folder, tol, what, close_calls=0.0):
 
 # 32-bit differs from the 64-bit plain statement by the rounding of a few hundred terms per sum, which the tests' wide
 # weights, their peaked softmaxes and the layers that run several times pass on (measured: one row in 400 reaches 5e-5);
-# bfloat16 rounds every stored activation to 8 bits
-TOL = {"float32": 1e-4, "bfloat16": 6e-2}
-CLOSE = {"float32": 0.0, "bfloat16": 0.08}
+# bfloat16 rounds every stored activation to 8 bits, ten runs of layers deep in some of the tests' models; there a share
+# of the rows may miss the tolerance (a choice between two experts whose scores lie within rounding goes the other way, and
+# the rows that attend to that row follow), while the median row must stay within half of it: a mechanism that is wrong
+# moves nearly every row by far more
+TOL = {"float32": 1e-4, "bfloat16": 8e-2}
+CLOSE = {"float32": 0.0, "bfloat16": 0.3}
 
 
 class _Step:
@@ -548,28 +553,28 @@ def drawn_config(seed):
     """A configuration drawn at random."""
     rng = np.random.RandomState(seed)
     pick = lambda *xs: xs[rng.randint(len(xs))]
-    width = int(pick(24, 40, 52, 64, 96, 136))
+    width = int(pick(24, 40, 50, 52, 64, 66, 96, 136, 75))
     layers = []
     n = int(rng.randint(1, 5))
     for _ in range(n):
         kind = rng.rand()
-        mlp = None if kind < 0.2 else DENSE(int(pick(16, 36, 64, 100))) if kind < 0.5 else \
-            MOE(int(pick(2, 3, 8, 11)), 1, int(pick(8, 12, 40)), shared=pick(None, 8, 24))
+        mlp = None if kind < 0.2 else DENSE(int(pick(16, 36, 37, 64, 100))) if kind < 0.5 else \
+            MOE(int(pick(1, 2, 3, 8, 11, 40)), 1, int(pick(8, 12, 13, 40)), shared=pick(None, 8, 9, 24))
         if mlp is not None and mlp["kind"] == "moe":
             mlp["router"]["top"] = int(rng.randint(1, mlp["router"]["experts"] + 1))
         kv = int(pick(1, 2, 3))
-        dim = int(pick(4, 8, 12, 16, 32, 56))
-        dims = int(pick(2, 4, dim))
+        dim = int(pick(4, 7, 8, 12, 16, 32, 56, 72))
+        dims = int(pick(2, 4, dim - dim % 2))
         rot = pick(None, ROT(float(pick(10.0, 1e3, 2.5e5)), dims, pick(None, (float(pick(2.0, 8.0)), 1.0, float(pick(2.0, 4.0)), int(pick(16, 64, 512))))))
-        layers.append((AT(kv * int(rng.randint(1, 4)), kv, dim, int(pick(4, 8, 20, 32, 48)), float(pick(0.1, 0.25, 0.5)),
-                          conv=pick(None, 1, 2, 4, 7), rot=rot), mlp))
+        layers.append((AT(kv * int(rng.randint(1, 4)), kv, dim, int(pick(4, 5, 8, 20, 32, 48, 80)), float(pick(0.1, 0.25, 0.5)),
+                          conv=pick(None, 1, 2, 4, 7, 16), rot=rot), mlp))
     start = int(rng.randint(0, n))
     loop = pick(None, (start, int(rng.randint(start + 1, n + 1)), int(rng.randint(1, 4))))
     return config(width, int(pick(50, 128, 301)), layers, loop=loop, eps=float(pick(1e-6, 1e-5, 1e-4)))
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("seed", range(8))
+@pytest.mark.parametrize("seed", range(16))
 def test_configurations_drawn_at_random(tmp_path, seed, dtype):
     cfg = drawn_config(seed)
     folder = make_folder(tmp_path / "m", cfg, seed=seed, edit=sharpen)
@@ -581,7 +586,9 @@ def test_configurations_drawn_at_random(tmp_path, seed, dtype):
                         ("mixed", H.steps_mixed(reqs, max_live=3, seed=seed))):
         got = H.run_steps(runner, steps)
         runner.cache.check()
-        compare(got, reqs, folder, TOL[dtype], "drawn configuration %d (%s) %s %s" % (seed, json.dumps(cfg), dtype, what), CLOSE[dtype])
+        # the drawn models go up to ten runs deep with up to 40 experts to choose from: more rows meet a close call
+        compare(got, reqs, folder, TOL[dtype], "drawn configuration %d (%s) %s %s" % (seed, json.dumps(cfg), dtype, what),
+                min(1.0, 2 * CLOSE[dtype]), median=1.0)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
