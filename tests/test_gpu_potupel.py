@@ -639,6 +639,46 @@ def test_a_far_key_decides_the_last_token(tmp_path, dtype):
         assert H.rel_err(plain(folder, moved)[-1], plain(folder, ids)[-1]) > 0.05      # the key matters in the plain statement
 
 
+LARGER = config(384, 1000, [
+    (AT(6, 2, 80, 48, 0.11, conv=3, rot=ROT(250000.0, 32, (8.0, 1.0, 4.0, 256))), DENSE(512)),
+    (AT(12, 4, 32, 32, 0.18, conv=4, rot=ROT(10000.0, 32)), MOE(16, 4, 64, shared=96)),
+    (AT(6, 6, 48, 80, 0.14, conv=2, rot=ROT(250000.0, 16, (4.0, 1.0, 2.0, 128))), MOE(6, 2, 128)),
+    (AT(3, 1, 128, 64, 0.09, conv=4, rot=ROT(500.0, 64)), DENSE(640)),
+], loop=(1, 3, 2), eps=1e-6)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_long_prompt_at_larger_sizes(tmp_path, dtype):
+    """1,300 tokens at once (the kernels for long portions, products of many rows), then 30 decoded tokens and a second
+    request in portions beside them; the last rows see keys a thousand tokens back."""
+    folder = make_folder(tmp_path / "m", LARGER, seed=11, std_scale=2.0, edit=sharpen)
+    reqs = {"long": H.random_tokens(1330, 1000, 1), "short": H.random_tokens(150, 1000, 2)}
+    from ginfer_amd import ModelRunner, StepEntry
+    runner = ModelRunner(folder, dtype=dtype, page_size=16, num_pages=-(-1600 // 16), max_requests=4, max_model_len=1600)
+    got = {}
+    logits = runner.step([StepEntry("long", reqs["long"][:1300], [0, 1, 640, 1299])]).cpu().numpy()
+    got.update({("long", p): row for p, row in zip([0, 1, 640, 1299], logits)})
+    at = 0
+    for k in range(30):
+        n = min(7, 150 - at)
+        entries = [StepEntry("long", reqs["long"][1300 + k:1301 + k], [0])] + ([StepEntry("short", reqs["short"][at:at + n], [n - 1])] if n else [])
+        logits = runner.step(entries).cpu().numpy()
+        got[("long", 1300 + k)] = logits[0]
+        if n:
+            got[("short", at + n - 1)] = logits[1]
+            at += n
+    runner.cache.check()
+    worst = []
+    for (rid, p), row in sorted(got.items()):
+        ref = plain(folder, reqs[rid])
+        worst.append(float(np.abs(row.astype(np.float64) - ref[p]).max() / np.abs(ref).max()))
+    assert np.isfinite(worst).all()
+    if dtype == "float32":
+        assert max(worst) < TOL[dtype], worst
+    else:
+        assert float(np.median(worst)) < TOL[dtype] / 2 and sum(w > TOL[dtype] for w in worst) <= CLOSE[dtype] * len(worst), worst
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_recorded_steps_equal_launched_ones(folders, dtype):
     reqs = requests_for("wide", [60, 25, 41], seed=80)
