@@ -123,14 +123,23 @@ class OutputNormBlock(Arrangement):
         return None
 
 
+class NormedRows:
+    """What a block hands to the next one in place of a pending delta when it has already added its own output into the
+    stream and made the rows of the next block's first norm in the same launch."""
+
+    def __init__(self, rows):
+        self.rows = rows
+
+
 @register_arrangement("sandwich")
 class SandwichBlock(Arrangement):
     """x <- x + out_norm1(mixer(norm1(x)));  x <- x + out_norm2(feed_forward(norm2(x))): a norm in front of every
     sublayer and one on its output (which may bring a factor per channel along).  A layer may have no feed-forward (then
     it has neither of that sublayer's norms).  The output norms are of a kind that offers `add_normed(residual, y,
     then)`; the norm in front of the feed-forward is handed to the mixer's output norm as `then`, so that one launch
-    adds the mixer's result and makes the rows the feed-forward reads.  The 32-bit stream is updated in place; nothing
-    is left pending for the next block."""
+    adds the mixer's result and makes the rows the feed-forward reads; in the same way the block's last output norm
+    makes the rows of the NEXT block's first norm where the model hands that norm over (`into_norm`; the next block then
+    gets `NormedRows` in place of a delta).  The 32-bit stream is updated in place; nothing is left pending."""
 
     roles = {"mixer": "mixer", "mixer_norm": "norm", "mixer_out_norm": "norm", "feed_forward": "feed_forward",
              "feed_forward_norm": "norm", "feed_forward_out_norm": "norm"}
@@ -149,22 +158,36 @@ class SandwichBlock(Arrangement):
                 raise ValueError("the output norms of this block add into the stream: %s has no add_normed"
                                  % type(norm).__name__)
         # the rows of the second norm come out of the first output norm's launch where that norm is a plain gain
-        self._fused_second = self.feed_forward_norm is not None and hasattr(self.feed_forward_norm, "weight") \
-            and hasattr(self.feed_forward_norm, "eps") and not getattr(self.feed_forward_norm, "has_bias", False)
+        self._fused_second = self.feed_forward_norm is not None and self._plain_gain(self.feed_forward_norm)
 
-    def forward(self, residual, delta, step, cache):
-        n = self.mixer_norm.forward(residual, whole(delta, self.mixer_norm))
+    @staticmethod
+    def _plain_gain(norm):
+        """Whether an output norm's launch can make this norm's rows: a gain per channel over the root mean square."""
+        return hasattr(norm, "weight") and hasattr(norm, "eps") and getattr(norm, "size", None) is not None \
+            and not getattr(norm, "has_bias", False) and type(norm).__name__ == "RMSNorm"
+
+    folds_output = True              # forward() takes `into_norm`
+
+    def takes_folded_input(self):
+        """The norm whose rows this block takes ready-made (NormedRows) in place of a delta, or None."""
+        return self.mixer_norm if self._plain_gain(self.mixer_norm) else None
+
+    def forward(self, residual, delta, step, cache, into_norm=None):
+        if isinstance(delta, NormedRows):           # the block before has made this block's first rows
+            n = delta.rows
+        else:
+            n = self.mixer_norm.forward(residual, whole(delta, self.mixer_norm))
         m = self.mixer.forward(n, step, cache)
         if self.feed_forward is None:
-            self.mixer_out_norm.add_normed(residual, m)
-            return None
+            rows = self.mixer_out_norm.add_normed(residual, m, then=into_norm)
+            return NormedRows(rows) if into_norm is not None else None
         if self._fused_second:
             n = self.mixer_out_norm.add_normed(residual, m, then=self.feed_forward_norm)
         else:
             self.mixer_out_norm.add_normed(residual, m)
             n = self.feed_forward_norm.forward(residual, None)
-        self.feed_forward_out_norm.add_normed(residual, self.feed_forward.forward(n))
-        return None
+        rows = self.feed_forward_out_norm.add_normed(residual, self.feed_forward.forward(n), then=into_norm)
+        return NormedRows(rows) if into_norm is not None else None
 
 
 def whole(delta, norm=None):

@@ -94,6 +94,8 @@ class DecoderModel:
             norm = takes() if takes is not None else None
             if i + 1 < len(self.schedule) and self.schedule[i + 1].enter:
                 norm = None                  # the stream changes between the two runs
+            if nxt is not None and type(nxt) is not type(self.blocks[e.layer]):
+                norm = None                  # what is handed over is the arrangement's own matter
             self._fold_into.append(norm if getattr(self.blocks[e.layer], "folds_output", False) else None)
 
     def _build(self, role, part_spec):
@@ -189,7 +191,7 @@ class DecoderModel:
     def _settle(residual, delta):
         """Adds what a block left pending into the stream."""
         if delta is not None:
-            if isinstance(delta, ops.ScaledRows):
+            if not isinstance(delta, torch.Tensor):
                 raise ValueError("a block that folds its output into the next block's norm cannot stand before a re-entry")
             residual.add_(whole(delta).to(residual.dtype))
         return None
